@@ -117,7 +117,11 @@ typedef struct qie_engine_opts {
                                 block-scaled fp8 MFMA (QIE_LINEAR_ACT_FP8) — activations
                                 quantised per row to e4m3 before each projection, a
                                 different model from the bf16-activation one (numerics flag) */
-    int32_t reserved[5];
+    int32_t compute_f32;     /* layered engines: 1 = every product, activation and cache row in
+                                true fp32 (weights widened exactly from bf16); 0 = bf16 matrix
+                                operands with fp32 accumulation, the residual stream, norms,
+                                routers, scores and softmax in fp32 either way               */
+    int32_t reserved[4];
 } qie_engine_opts;
 
 int qie_engine_create(const qie_model_spec* spec, const qie_engine_opts* opts, qie_engine** out);
@@ -238,6 +242,82 @@ int qie_batch_time_kernel(qie_batch* b, int32_t which, int32_t iters, double* av
  * 2l + 1 = after layer l's attention block (O-proj + residual), 2l + 2 = after its MLP
  * block (down-proj + residual).  Parity diagnostics (tools/flip_attrib.py). */
 int qie_batch_debug_step(qie_batch* b, const qie_sampling* smp, int32_t* next_ids, void* host_x);
+
+
+/* ---------------------------------------------------------- layered engines
+ * A model given as a per-layer program instead of the fixed Qwen decoder: every layer names its
+ * mixer and its feed-forward with their own sizes and constants, so one engine serves layer
+ * orders and sizes that differ from layer to layer.  The same qie_engine / qie_batch handles,
+ * slots, block table and page pool as above; the step is ragged (qie_batch_step): portions of
+ * prompts beside single decoded tokens in one pass.
+ *
+ * Mixer QIE_MIXER_LATENT_ATTENTION: queries q = W_q h laid out per head as [dim unrotated |
+ * rot_dim rotated]; W_dkv h = [compressed row (kv_rank), RMS-normed with a weight | one rotated
+ * key part shared by all heads]; per head k = W_uk c, v = W_uv c; rotate-half rotary on the
+ * first rot_dims coordinates of the rotated parts (angle pos * rot_base^(-2i/rot_dims));
+ * softmax over the last `window` positions; per-head sigmoid gate from the mixer's input;
+ * W_o.  Only [c | rotated key part] is cached.  kv_from >= 0: the layer has no W_dkv and reads
+ * that layer's cache rows.  The engine runs the absorbed form (W_uk folded into the query,
+ * W_uv applied to the softmax-weighted sum of c), for prompts and decoding alike.
+ * Feed-forward: none, dense gated SiLU, or a mixture of `experts` gated-SiLU experts with a
+ * sigmoid router (fp32) whose `top` largest scores, not renormalised, scale the experts' input.
+ * Layer: y = x + g1 * rms(mixer(x)); z = y + g2 * rms(ff(y)) (scalar gains, norm on the
+ * sublayer's output); the next layer's input is the depth-weighted sum over the embedding
+ * output and every layer result so far. */
+enum { QIE_MIXER_LATENT_ATTENTION = 1 };
+enum { QIE_FF_NONE = 0, QIE_FF_DENSE = 1, QIE_FF_MOE = 2 };
+
+typedef struct qie_layer_desc {
+    int32_t mixer;            /* QIE_MIXER_*                                          */
+    int32_t heads, dim, rot_dim, vdim, kv_rank;
+    int32_t window;           /* position i sees j with 0 <= i - j < window           */
+    int32_t kv_from;          /* -1: own W_dkv; else the layer whose cache rows it reads */
+    int32_t rot_dims;         /* rotated coordinates of a rotated part (even, <= rot_dim) */
+    float rot_base, scale;
+    int32_t ff_kind;          /* QIE_FF_*                                             */
+    int32_t ff;               /* hidden size of the dense feed-forward / of one expert */
+    int32_t experts, top;
+    int32_t reserved[4];
+} qie_layer_desc;
+
+typedef struct qie_arch_desc {
+    int32_t n_layers, width, vocab;
+    float norm_eps;
+    int32_t depth_mix;        /* 1: depth-weighted sum of all earlier results ('l<i>.dwa') */
+    int32_t reserved[7];
+    const qie_layer_desc* layers;
+} qie_arch_desc;
+
+int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* opts, qie_engine** out);
+/* Hand the engine one checkpoint tensor (host memory, copied): dtype 0 = bf16 words, 1 = int32,
+ * 2 = fp32.  Names: 'embed', 'head', 'final.norm', 'l<i>.norm1|norm2|dwa',
+ * 'l<i>.mix.q|dkv|dkv.norm|uk|uv|g|o', 'l<i>.mlp.gate|up|down|router', 'l<i>.mlp.e<j>.gate|up|down'.
+ * qie_engine_finalize_weights checks every tensor the architecture needs against its shape,
+ * builds the device layouts (fused projection rows, per-head transposed W_uk, experts end to
+ * end) and drops the host copies. */
+int qie_engine_put_tensor(qie_engine* e, const char* name, const void* host, int32_t dtype, int32_t ndim,
+                          const int64_t* shape);
+int qie_engine_finalize_weights(qie_engine* e);
+/* One ragged step over a paged batch of a layered engine (qie_batch_create_paged; page_tokens a
+ * power of two >= 16): entry i feeds counts[i] tokens (laid end to end in `tokens`) to slot
+ * slots[i], continuing at the slot's position (a released or fresh slot starts at 0).  Pages are
+ * taken for exactly the positions written, all-or-nothing over the whole step.  want_rows
+ * (n_want indices into the step's packed rows) selects the rows whose logits are computed:
+ * fp32 [n_want][vocab] to host_logits (may be NULL: they stay on the device for
+ * qie_batch_step_sample). */
+int qie_batch_step(qie_batch* b, int32_t n_entries, const int32_t* slots, const int32_t* counts, const int32_t* tokens,
+                   int32_t n_want, const int32_t* want_rows, float* host_logits);
+/* Samples one id per wanted row of the last qie_batch_step (qie_sample on the rows, rounded to
+ * bf16 as the sampler reads them); host_ids [n_want]. */
+int qie_batch_step_sample(qie_batch* b, const qie_sampling* s, int32_t* host_ids);
+/* Diagnostics: enable != 0 makes every following step keep the stream after each layer;
+ * qie_batch_step_layers copies the last step's [n_layers][rows][width] fp32 to host_out. */
+int qie_batch_keep_layers(qie_batch* b, int32_t enable);
+int qie_batch_step_layers(qie_batch* b, float* host_out, int64_t n);
+/* Time `iters` runs of one stage of the last step's shape (hipEvents on the engine stream):
+ * which 0 = the whole layer stack, 1 = attention of `layer`, 2 = its projections (input, absorb,
+ * value expansion, output), 3 = its feed-forward.  The cache is read, not advanced. */
+int qie_batch_time_stage(qie_batch* b, int32_t which, int32_t layer, int32_t iters, double* avg_us);
 
 #ifdef __cplusplus
 }

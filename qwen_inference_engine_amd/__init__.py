@@ -6,6 +6,7 @@ kernels in libqie.so behind a C ABI (include/qie/*.h), driven from C++ or from t
 thin Python layer.  See DESIGN.md.
 """
 from .spec import ModelSpec, PRESETS, QWEN2_0_5B, QWEN2_7B, QWEN2_72B, QWEN3_14B, tiny  # noqa: F401
+from .spec import LayeredSpec, LatentAttention, FeedForward, LayerSpec, ARCHITECTURES, spec_from_config, spec_from_dir  # noqa: F401
 from .weights import HostWeights, SynthParams, synthetic_index, parse_meta, format_meta  # noqa: F401
 from .engine import Engine, Batch, Comm, Sampling, GREEDY  # noqa: F401
 

@@ -78,7 +78,24 @@ class EngineOptsC(C.Structure):
     _fields_ = [("device", C.c_int32), ("max_ctx", C.c_int32), ("use_graph", C.c_int32),
                 ("tp_rank", C.c_int32), ("tp_size", C.c_int32), ("tp_comm", C.c_void_p),
                 ("weight_fp8", C.c_int32), ("comm_always", C.c_int32), ("prefill_fp8", C.c_int32),
-                ("reserved", C.c_int32 * 5)]
+                ("compute_f32", C.c_int32), ("reserved", C.c_int32 * 4)]
+
+
+QIE_MIXER_LATENT_ATTENTION = 1
+QIE_FF_NONE, QIE_FF_DENSE, QIE_FF_MOE = 0, 1, 2
+
+
+class LayerDescC(C.Structure):
+    _fields_ = [("mixer", C.c_int32), ("heads", C.c_int32), ("dim", C.c_int32), ("rot_dim", C.c_int32),
+                ("vdim", C.c_int32), ("kv_rank", C.c_int32), ("window", C.c_int32), ("kv_from", C.c_int32),
+                ("rot_dims", C.c_int32), ("rot_base", C.c_float), ("scale", C.c_float),
+                ("ff_kind", C.c_int32), ("ff", C.c_int32), ("experts", C.c_int32), ("top", C.c_int32),
+                ("reserved", C.c_int32 * 4)]
+
+
+class ArchDescC(C.Structure):
+    _fields_ = [("n_layers", C.c_int32), ("width", C.c_int32), ("vocab", C.c_int32), ("norm_eps", C.c_float),
+                ("depth_mix", C.c_int32), ("reserved", C.c_int32 * 7), ("layers", C.POINTER(LayerDescC))]
 
 
 # (name, restype, argtypes) — every symbol the public headers declare.
@@ -196,6 +213,14 @@ SIGNATURES = [
     ("qie_engine_rope_tables", C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), _PI32]),
     ("qie_batch_time_kernel", C.c_int, [_P, _I32, _I32, _PD, _PD]),
     ("qie_batch_debug_step", C.c_int, [_P, _P, _PI32, _P]),
+    ("qie_engine_create_layered", C.c_int, [C.POINTER(ArchDescC), C.POINTER(EngineOptsC), C.POINTER(_P)]),
+    ("qie_engine_put_tensor", C.c_int, [_P, C.c_char_p, _P, _I32, _I32, _PI64]),
+    ("qie_engine_finalize_weights", C.c_int, [_P]),
+    ("qie_batch_step", C.c_int, [_P, _I32, _PI32, _PI32, _PI32, _I32, _PI32, _PF]),
+    ("qie_batch_step_sample", C.c_int, [_P, C.POINTER(SamplingC), _PI32]),
+    ("qie_batch_keep_layers", C.c_int, [_P, _I32]),
+    ("qie_batch_step_layers", C.c_int, [_P, _PF, _I64]),
+    ("qie_batch_time_stage", C.c_int, [_P, _I32, _I32, _I32, _PD]),
 ]
 
 _lib = None

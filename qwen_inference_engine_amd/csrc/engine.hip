@@ -14,10 +14,7 @@
 // plus [rms+lm_head GEMV + fused arg-max] [finalize: id, position, next
 // embedding], captured once into a hipGraph; positions and token ids live in
 // device memory so the graph replays without host edits.
-#include "qie_common.hpp"
-#include "../../include/qie/qie_engine.h"
-#include "qie_index.hpp"
-#include "qie_comm.hpp"
+#include "engine_impl.hpp"
 
 #include <chrono>
 #include <cstring>
@@ -46,22 +43,6 @@ int persist_ts_slots();
 
 using namespace qie;
 
-// Tensor-parallel shard of one rank (tp = 1: the whole model).  Column-parallel
-// QKV (by heads) and gate/up (by I), row-parallel O and down, vocab-parallel lm_head;
-// embedding, norms and the residual stream are replicated.
-// Heads: n_kv_heads % tp == 0 splits both head kinds evenly; otherwise, when
-// tp % n_kv_heads == 0, every kv head is replicated on rep = tp / n_kv_heads ranks and
-// the G = n_heads / n_kv_heads q heads of its group are split among those ranks as
-// evenly as they go (the first G % rep ranks take one more): Qwen2-7B (28 / 4 heads) at
-// TP 8 gives q heads 4,3,4,3,... with one kv head each.  Every q head lives
-// on exactly one rank, so the row-parallel O all-reduce still sums each head once.
-struct TpShard {
-    int tp = 1, rank = 0;
-    int nq = 0, nkv = 0, ffn = 0, vocab = 0;   // local counts
-    int q0 = 0, kv0 = 0;                        // first global q / kv head of this rank
-    int64_t vocab0 = 0;                         // first global vocab row of this rank
-};
-
 // Head split of rank `rank` of `tp` (see TpShard); false when the heads do not shard.
 static bool shard_heads(int nq, int nkv, int tp, int rank, TpShard& sh) {
     if (nkv % tp == 0 && nq % tp == 0) {
@@ -81,92 +62,6 @@ static bool shard_heads(int nq, int nkv, int tp, int rank, TpShard& sh) {
     sh.q0 = g * G + sub * base + std::min(sub, extra);
     return true;
 }
-
-struct qie_engine {
-    qie_model_spec spec{};   // the full model
-    TpShard sh;              // this rank's shard
-    qie_comm* comm = nullptr;
-    qie_engine_opts opts{};
-    hipStream_t stream = nullptr;
-    void* arena = nullptr;
-    size_t arena_bytes = 0;
-    qie_index* index = nullptr;
-    std::vector<qie_layer_weights> layers;
-    qie_model_weights w{};
-    bool have_weights = false;
-    bool fp8 = false;            // linear weights are e4m3 + row scales (fp8_arena)
-    bool fp8_t16 = false;        // ... and the decode projections in the 16-row tiled layout
-    bool fp8_t16_head = false;   // ... and the lm_head too
-    // fp8 engines: the same (dequantised) layer weights as bf16, in place in the arena —
-    // prefill's MFMA GEMMs read these (compute-bound: the LDS-DMA bf16 kernel), decode's
-    // bandwidth-bound GEMVs the fp8 codes; both compute the one dequantised model
-    std::vector<qie_layer_weights> layers_pf;
-    void* fp8_arena = nullptr;
-    float* rope_cos = nullptr;
-    float* rope_sin = nullptr;
-    int rope_rows = 0;
-};
-
-struct qie_batch {
-    qie_engine* e = nullptr;
-    int B = 0, max_ctx = 0;
-    uint16_t* kc = nullptr;
-    uint16_t* vc = nullptr;
-    int64_t seq_stride = 0;
-    int run_pad = 0;             // contiguous: run = max_ctx + run_pad tokens (dev A/B)
-    int32_t* d_pos = nullptr;
-    float* d_rope_cur = nullptr;   // [B][rope_cur_stride(hd)]: RoPE row of each slot's current position
-    int32_t* d_step = nullptr;
-    int32_t* d_hist = nullptr;
-    int32_t* d_ids = nullptr;
-    unsigned long long* d_keys = nullptr;
-    uint16_t* x_res = nullptr;
-    uint16_t* qkv = nullptr;
-    uint16_t* q = nullptr;
-    uint16_t* att = nullptr;
-    uint16_t* h = nullptr;
-    uint16_t* xn = nullptr;     // [B][H] RMS-normed rows feeding the batched (B >= 2) projections
-    uint16_t* logits = nullptr;
-    void* attn_ws = nullptr;
-    void* dec_ws = nullptr;     // fused decode attention: split partials + zeroed counters
-    void* samp_ws = nullptr;
-    // tensor parallel: fp32 partials of the row-parallel projections, gathered logits
-    float* part = nullptr;            // [B][H]
-    uint16_t* logits_full = nullptr;  // [B][V]
-    uint16_t* gather_tmp = nullptr;   // [tp][B][V/tp]
-    float* pf_part = nullptr;         // [pf_rows][H]
-    std::vector<int32_t> h_pos;
-    // prefill scratch
-    int64_t pf_rows = 0;
-    uint16_t *pf_x = nullptr, *pf_hn = nullptr, *pf_qkv = nullptr, *pf_q = nullptr, *pf_att = nullptr,
-             *pf_h = nullptr;
-    int32_t *pf_pos = nullptr, *pf_ids = nullptr;
-    uint8_t *pf_q8 = nullptr, *pf_e8 = nullptr;   // fp8 prefill (opts.prefill_fp8): codes [rows][max K], exps [rows]
-    void* pf_attn_ws = nullptr;
-    int64_t pf_attn_ws_bytes = 0;   // the split workspace depends on n (short prompts split), not on n <= pf_rows
-    // paged KV (qie_batch_create_paged): pool pages of page_tokens tokens, block table
-    // [B][max_pages] on device and host, free list, pages held per slot
-    int page_tokens = 0, max_pages = 0, n_pages = 0;
-    int32_t* d_table = nullptr;
-    std::vector<int32_t> h_table, free_pages, held;
-    std::vector<char> idle;
-    bool table_dirty = false;
-    // decode graph
-    hipGraphExec_t gexec = nullptr;
-    qie_sampling gs{};
-    bool graph_ok = false;
-    // qie_batch_debug_step: while set, the decode enqueue copies the residual stream after every
-    // attention block and every MLP block into dbg_x ([2L + 1][B][H] bf16; slot 0 = the input)
-    uint16_t* dbg_x = nullptr;
-    // decode structure (qie_batch_set_decode_mode): 0 = five launches per layer, 1 = the whole
-    // layer stack as one persistent launch (k_persist.hip).  pk_mem: hand-off granules, then the
-    // step epoch and the error word (zeroed once; the finalize kernel advances the epoch)
-    int decode_mode = 0;
-    void* pk_mem = nullptr;
-    qie_layer_weights* d_layers = nullptr;
-    void* d_attp = nullptr;      // the attention role's parameters per layer (persist_attn_table)
-    unsigned long long* pk_ts = nullptr;   // qie_batch_pk_trace: phase timestamps [cu][layer][slots]
-};
 
 namespace qie {
 
@@ -245,7 +140,7 @@ __global__ void copy_ids_kernel(const int32_t* src, int32_t* dst, int len, int64
     if (i < len) dst[blockIdx.y * dst_stride + i] = src[(int64_t)blockIdx.y * len + i];
 }
 
-static int dmalloc(void** p, size_t bytes) {
+int dmalloc(void** p, size_t bytes) {
     QIE_HIP(hipMalloc(p, bytes < 16 ? 16 : bytes));
     return 0;
 }
@@ -280,7 +175,7 @@ static qie_kv_cache batch_cache(const qie_batch* b, int seq0) {
 // ------------------------------------------------------------ page pool
 // Host-side allocator of the paged batch.  Decisions are deterministic, so the
 // tensor-parallel ranks (each holding its own heads' pages) stay in step.
-static int ensure_pages(qie_batch* b, int seq, int64_t ntok) {
+int ensure_pages(qie_batch* b, int seq, int64_t ntok) {
     if (!b->d_table) return 0;
     const int64_t need = (ntok + b->page_tokens - 1) / b->page_tokens;
     QIE_REQUIRE(need <= b->max_pages, "KV pages: %lld tokens exceed max_ctx %d", (long long)ntok, b->max_ctx);
@@ -295,7 +190,7 @@ static int ensure_pages(qie_batch* b, int seq, int64_t ntok) {
     return 0;
 }
 
-static void drop_pages(qie_batch* b, int seq) {
+void drop_pages(qie_batch* b, int seq) {
     if (!b->d_table) return;
     for (int i = b->held[seq] - 1; i >= 0; i--) {
         int32_t& t = b->h_table[(int64_t)seq * b->max_pages + i];
@@ -307,7 +202,7 @@ static void drop_pages(qie_batch* b, int seq) {
 }
 
 // uploads the host table (ordered after everything already on the stream)
-static int flush_table(qie_batch* b) {
+int flush_table(qie_batch* b) {
     if (!b->d_table || !b->table_dirty) return 0;
     // on the engine stream (non-blocking: a legacy-null-stream copy is not ordered before its
     // kernels), complete before the host table may change again
@@ -988,6 +883,7 @@ static int init_synthetic_sharded(qie_engine* e, uint64_t seed, float w_scale, f
 }
 
 int qie_engine_init_synthetic(qie_engine* e, uint64_t seed, float w_scale, float norm_scale, float bias_scale) {
+    QIE_REQUIRE(!e || !e->lm, "%s: a layered engine takes its tensors through qie_engine_put_tensor", __func__);
     QIE_REQUIRE(e, "qie_engine_init_synthetic: null engine");
     if (e->sh.tp > 1) return init_synthetic_sharded(e, seed, w_scale, norm_scale, bias_scale);
     QIE_TRY(alloc_arena_synthetic(e));
@@ -1061,6 +957,7 @@ static int load_weights_sharded(qie_engine* e, const char* weights_bin, const ch
 }
 
 int qie_engine_load_weights_bin(qie_engine* e, const char* weights_bin, const char* meta, int64_t chunk_bytes) {
+    QIE_REQUIRE(!e || !e->lm, "%s: a layered engine takes its tensors through qie_engine_put_tensor", __func__);
     QIE_REQUIRE(e && weights_bin && meta, "qie_engine_load_weights_bin: bad arguments");
     if (e->sh.tp > 1) return load_weights_sharded(e, weights_bin, meta);
     if (e->index) qie_index_destroy(e->index);
@@ -1114,6 +1011,7 @@ int qie_engine_load_weights_bin(qie_engine* e, const char* weights_bin, const ch
 }
 
 int qie_engine_set_weights(qie_engine* e, const qie_model_weights* w) {
+    QIE_REQUIRE(!e || !e->lm, "%s: a layered engine takes its tensors through qie_engine_put_tensor", __func__);
     QIE_REQUIRE(e && w && w->layers && w->n_layers == e->spec.n_layers && w->embed && w->final_norm && w->lm_head,
                 "qie_engine_set_weights: bad arguments");
     e->layers.assign(w->layers, w->layers + w->n_layers);
@@ -1133,6 +1031,7 @@ int qie_engine_set_weights(qie_engine* e, const qie_model_weights* w) {
 }
 
 int qie_engine_weights(const qie_engine* e, qie_model_weights* out, const qie_layer_weights** layers) {
+    QIE_REQUIRE(!e || !e->lm, "%s: a layered engine takes its tensors through qie_engine_put_tensor", __func__);
     QIE_REQUIRE(e && e->have_weights, "qie_engine_weights: no weights");
     if (out) *out = e->w;
     if (layers) *layers = e->layers.data();
@@ -1156,6 +1055,7 @@ int qie_engine_sync(qie_engine* e) {
 void qie_engine_destroy(qie_engine* e) {
     if (!e) return;
     if (e->stream) hipStreamSynchronize(e->stream);
+    layered_engine_destroy(e);
     if (e->arena) hipFree(e->arena);
     if (e->fp8_arena) hipFree(e->fp8_arena);
     if (e->rope_cos) hipFree(e->rope_cos);
@@ -1256,11 +1156,13 @@ static int batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t p
 }
 
 int qie_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, qie_batch** out) {
+    QIE_REQUIRE(!e || !e->lm, "qie_batch_create: a layered engine takes a paged batch (qie_batch_create_paged)");
     return batch_create(e, batch, max_ctx, 0, 0, out);
 }
 
 int qie_batch_create_paged(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t page_tokens, int32_t n_pages,
                            qie_batch** out) {
+    if (e && e->lm) return layered_batch_create(e, batch, max_ctx, page_tokens, n_pages, out);
     if (page_tokens == 0) page_tokens = 128;
     QIE_REQUIRE(page_tokens >= 128 && (page_tokens & (page_tokens - 1)) == 0,
                 "qie_batch_create_paged: page_tokens %d must be a power of two >= 128", page_tokens);
@@ -1275,6 +1177,10 @@ int qie_batch_release(qie_batch* b, int32_t seq) {
     b->idle[seq] = 1;
     QIE_TRY(flush_table(b));
     qie_engine* e = b->e;
+    if (b->lb) {   // a layered batch keeps no per-slot device state beside the table
+        b->h_pos[seq] = 0;
+        return 0;
+    }
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(256), 0, e->stream, seq, 0, 0, 0, b->d_pos, b->d_step, b->d_hist,
                        b->max_ctx, (const uint4*)e->w.embed, (uint4*)b->x_res, (int64_t)e->spec.hidden / 8, 1, rope_cur_args(b));
     QIE_LAUNCH_CHECK();
@@ -1304,6 +1210,7 @@ void qie_batch_destroy(qie_batch* b) {
     if (!b) return;
     if (b->e && b->e->stream) hipStreamSynchronize(b->e->stream);
     if (b->gexec) hipGraphExecDestroy(b->gexec);
+    layered_batch_destroy(b);
     void* ps[] = {b->kc, b->vc, b->d_table, b->d_pos, b->d_rope_cur, b->d_step, b->d_hist, b->d_ids, b->d_keys, b->x_res, b->qkv, b->q,
                   b->att, b->h, b->logits, b->attn_ws, b->dec_ws, b->samp_ws, b->pf_x, b->pf_hn, b->pf_qkv, b->pf_q,
                   b->pf_att, b->pf_h, b->pf_pos, b->pf_ids, b->pf_attn_ws, b->part, b->logits_full,
@@ -1455,11 +1362,13 @@ static int prefill_rows(qie_batch* b, int seq0, int n_seqs, const int32_t* ids, 
 }
 
 int qie_prefill(qie_batch* b, int32_t seq, const int32_t* ids, int32_t n, const qie_sampling* smp, int32_t* next_id) {
+    QIE_REQUIRE(!b || !b->lb, "%s: not for a batch of a layered engine (qie_batch_step drives it)", __func__);
     return prefill_rows(b, seq, 1, ids, n, smp, next_id, "qie_prefill");
 }
 
 int qie_prefill_batch(qie_batch* b, int32_t seq0, int32_t n_seqs, const int32_t* ids, int32_t len,
                       const qie_sampling* smp, int32_t* next_ids) {
+    QIE_REQUIRE(!b || !b->lb, "%s: not for a batch of a layered engine (qie_batch_step drives it)", __func__);
     return prefill_rows(b, seq0, n_seqs, ids, len, smp, next_ids, "qie_prefill_batch");
 }
 
@@ -1550,6 +1459,7 @@ static int prepare_steps(qie_batch* b, int n_steps, const char* who) {
 }
 
 int qie_decode_step(qie_batch* b, const qie_sampling* smp, int32_t* next_ids) {
+    QIE_REQUIRE(!b || !b->lb, "%s: not for a batch of a layered engine (qie_batch_step drives it)", __func__);
     QIE_REQUIRE(b, "qie_decode_step: null batch");
     QIE_TRY(prepare_steps(b, 1, "qie_decode_step"));
     QIE_TRY(launch_step(b, smp));
@@ -1558,6 +1468,7 @@ int qie_decode_step(qie_batch* b, const qie_sampling* smp, int32_t* next_ids) {
 }
 
 int qie_decode(qie_batch* b, int32_t n_steps, const qie_sampling* smp, int32_t* out_ids) {
+    QIE_REQUIRE(!b || !b->lb, "%s: not for a batch of a layered engine (qie_batch_step drives it)", __func__);
     QIE_REQUIRE(b && n_steps >= 0, "qie_decode: bad arguments");
     QIE_TRY(prepare_steps(b, n_steps, "qie_decode"));
     std::vector<int32_t> p0 = b->h_pos;
@@ -1579,6 +1490,7 @@ int qie_decode(qie_batch* b, int32_t n_steps, const qie_sampling* smp, int32_t* 
 }
 
 int qie_batch_logits(qie_batch* b, void* host_out) {
+    QIE_REQUIRE(!b || !b->lb, "%s: not for a batch of a layered engine (qie_batch_step drives it)", __func__);
     QIE_REQUIRE(b && host_out, "qie_batch_logits: bad arguments");
     const uint16_t* src = b->logits;
     if (use_comm(b->e)) {   // collective: every rank calls this at the same point
@@ -1594,12 +1506,17 @@ int qie_batch_logits(qie_batch* b, void* host_out) {
 
 int qie_batch_positions(qie_batch* b, int32_t* host_pos) {
     QIE_REQUIRE(b && host_pos, "qie_batch_positions: bad arguments");
+    if (b->lb) {   // positions of a layered batch live on the host
+        for (int m = 0; m < b->B; m++) host_pos[m] = b->idle[m] ? 0 : b->h_pos[m];
+        return 0;
+    }
     QIE_HIP(hipStreamSynchronize(b->e->stream));
     QIE_HIP(d2h(b->e, host_pos, b->d_pos, (size_t)b->B * 4));
     return 0;
 }
 
 int qie_batch_history(qie_batch* b, int32_t seq, int32_t* host_ids, int32_t n) {
+    QIE_REQUIRE(!b || !b->lb, "%s: not for a batch of a layered engine (qie_batch_step drives it)", __func__);
     QIE_REQUIRE(b && host_ids && seq >= 0 && seq < b->B && n >= 0 && n <= b->max_ctx,
                 "qie_batch_history: bad arguments");
     QIE_HIP(hipStreamSynchronize(b->e->stream));
@@ -1608,6 +1525,7 @@ int qie_batch_history(qie_batch* b, int32_t seq, int32_t* host_ids, int32_t n) {
 }
 
 int qie_batch_set_position(qie_batch* b, int32_t seq, int32_t pos, int32_t token) {
+    QIE_REQUIRE(!b || !b->lb, "%s: not for a batch of a layered engine (qie_batch_step drives it)", __func__);
     QIE_REQUIRE(b && seq >= 0 && seq < b->B && pos >= 0 && pos + 1 < b->max_ctx && token >= 0 &&
                     token < b->e->spec.vocab,
                 "qie_batch_set_position: bad arguments");
@@ -1625,6 +1543,7 @@ int qie_batch_set_position(qie_batch* b, int32_t seq, int32_t pos, int32_t token
 }
 
 int qie_batch_set_decode_mode(qie_batch* b, int32_t mode) {
+    QIE_REQUIRE(!b || !b->lb, "%s: not for a batch of a layered engine (qie_batch_step drives it)", __func__);
     QIE_REQUIRE(b && (mode == 0 || mode == 1), "qie_batch_set_decode_mode: bad arguments (mode 0 or 1)");
     qie_engine* e = b->e;
     if (mode == 1) {
@@ -1671,6 +1590,7 @@ int qie_batch_set_decode_mode(qie_batch* b, int32_t mode) {
 int qie_batch_decode_mode(const qie_batch* b) { return b ? b->decode_mode : -22; }
 
 int qie_batch_pk_trace(qie_batch* b, int32_t enable, uint64_t* host_out, int64_t n) {
+    QIE_REQUIRE(!b || !b->lb, "%s: not for a batch of a layered engine (qie_batch_step drives it)", __func__);
     QIE_REQUIRE(b, "qie_batch_pk_trace: null batch");
     qie_engine* e = b->e;
     const int64_t need = (int64_t)device_cu_count() * e->spec.n_layers * persist_ts_slots();
@@ -1701,12 +1621,14 @@ int qie_batch_dims(const qie_batch* b, int32_t* batch, int32_t* max_ctx) {
 }
 
 int qie_batch_kv_cache(const qie_batch* b, int32_t seq, qie_kv_cache* out) {
+    QIE_REQUIRE(!b || !b->lb, "%s: not for a batch of a layered engine (qie_batch_step drives it)", __func__);
     QIE_REQUIRE(b && out && seq >= 0 && seq < b->B, "qie_batch_kv_cache: bad arguments");
     *out = batch_cache(b, seq);
     return 0;
 }
 
 int qie_batch_reserve(qie_batch* b, int32_t seq, int32_t n_tokens) {
+    QIE_REQUIRE(!b || !b->lb, "%s: not for a batch of a layered engine (qie_batch_step drives it)", __func__);
     QIE_REQUIRE(b && seq >= 0 && seq < b->B && n_tokens >= 0, "qie_batch_reserve: bad arguments");
     QIE_REQUIRE(n_tokens <= b->max_ctx, "qie_batch_reserve: %d tokens exceed max_ctx %d", n_tokens, b->max_ctx);
     QIE_TRY(ensure_pages(b, seq, n_tokens));
@@ -1794,6 +1716,7 @@ static int time_persistent(qie_batch* b, int iters, double* avg_us, double* byte
 }
 
 int qie_batch_time_kernel(qie_batch* b, int32_t which, int32_t iters, double* avg_us, double* bytes) {
+    QIE_REQUIRE(!b || !b->lb, "%s: not for a batch of a layered engine (qie_batch_step drives it)", __func__);
     QIE_REQUIRE(b && iters > 0 && avg_us && bytes && which >= 0 && which <= 6, "qie_batch_time_kernel: bad arguments");
     qie_engine* e = b->e;
     if (which == 6) return time_persistent(b, iters, avg_us, bytes);
@@ -1895,6 +1818,7 @@ int qie_batch_time_kernel(qie_batch* b, int32_t which, int32_t iters, double* av
 }
 
 int qie_batch_debug_step(qie_batch* b, const qie_sampling* smp, int32_t* next_ids, void* host_x) {
+    QIE_REQUIRE(!b || !b->lb, "%s: not for a batch of a layered engine (qie_batch_step drives it)", __func__);
     QIE_REQUIRE(b && host_x, "qie_batch_debug_step: bad arguments");
     qie_engine* e = b->e;
     const int64_t n = (int64_t)b->B * e->spec.hidden, slots = 2 * (int64_t)e->spec.n_layers + 1;

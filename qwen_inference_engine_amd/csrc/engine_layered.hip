@@ -1,0 +1,835 @@
+// engine_layered.hip — the engine tier for models given as a per-layer program
+// (qie_engine_create_layered, qie_engine_put_tensor, qie_batch_step; qie_engine.h).
+//
+// A layered engine is a qie_engine whose `lm` holds the architecture and the device weights; a
+// batch of it is a paged qie_batch whose pool holds latent cache rows instead of K / V rows and
+// whose `lb` holds the step's activations.  Slots, the block table and the page pool are the
+// batch's own (ensure_pages / drop_pages / flush_table, qie_batch_release, qie_batch_page_stats).
+//
+// A step packs the rows of all entries (portions of prompts and single tokens alike) end to
+// end; every projection runs once over all rows, the cache append and the attention address
+// their rows through (slot, position) pairs.  fp32: residual stream, norms, router, scores,
+// softmax, rotary angles (tables built in double on the host).  compute_f32 = 0 rounds matrix
+// operands to bf16 (weights are bf16, the cache rows are stored as bf16); = 1 keeps everything
+// fp32.
+#include "engine_impl.hpp"
+#include "k_layered.hpp"
+
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <string>
+
+namespace qie {
+
+struct HostTensor {
+    int dtype = 0;   // 0 bf16 words, 1 int32, 2 fp32
+    std::vector<int64_t> shape;
+    std::vector<uint8_t> data;
+    int64_t numel() const {
+        int64_t n = 1;
+        for (int64_t s : shape) n *= s;
+        return n;
+    }
+};
+
+struct RopeTab {
+    double base;
+    int dims;
+    float* cs;
+    float* sn;
+};
+
+struct LayerDev {
+    qie_layer_desc d{};
+    int cache_layer = 0;   // the layer whose cache rows this layer reads
+    int rope = 0;
+    void* w_in = nullptr;   // [q ; dkv ; g] rows (kv_from layers: [q ; g])
+    int n_in = 0, g_col = 0;
+    float* dkv_norm = nullptr;
+    void* uk_t = nullptr;   // [heads][kv_rank][dim]
+    void* uv = nullptr;     // [heads * vdim][kv_rank]
+    void* wo = nullptr;     // [width][heads * vdim]
+    float g1 = 1.f, g2 = 1.f;
+    void* w_gu = nullptr;     // dense [2 ff][width]; moe [experts][2 ff][width]
+    void* w_down = nullptr;   // dense [width][ff];   moe [experts][width][ff]
+    void* w_router = nullptr;
+    float* dwa = nullptr;     // [i + 2]
+};
+
+struct LayeredModel {
+    qie_arch_desc a{};
+    std::vector<qie_layer_desc> descs;
+    bool f32 = false;
+    std::map<std::string, HostTensor> host;
+    std::vector<LayerDev> L;
+    std::vector<RopeTab> ropes;
+    void* embed = nullptr;
+    void* head = nullptr;
+    float g_final = 1.f;
+    std::vector<void*> allocs;
+    bool final = false;
+    size_t esz() const { return f32 ? 4 : 2; }
+};
+
+struct LayeredBatch {
+    std::vector<int64_t> layer_off;   // element offset of each caching layer's rows inside a page
+    int64_t cap = 0, want_cap = 0;
+    float *stack = nullptr, *x = nullptr, *proj = nullptr, *qabs = nullptr, *olat = nullptr, *ov = nullptr, *mix = nullptr,
+          *y = nullptr, *gu = nullptr, *act = nullptr, *ffo = nullptr, *xg = nullptr, *yd = nullptr, *score = nullptr,
+          *xn = nullptr, *logits = nullptr, *keep = nullptr;
+    uint16_t* logits_bf = nullptr;
+    int32_t *row_slot = nullptr, *row_pos = nullptr, *tok = nullptr, *want = nullptr, *sel = nullptr, *cnt = nullptr,
+            *off = nullptr, *slot_of = nullptr, *d_ids = nullptr, *d_step = nullptr;
+    int32_t* h_stage = nullptr;   // pinned: row_slot, row_pos, tok of a step
+    int64_t h_stage_rows = 0;
+    int last_T = 0, last_want = 0;
+    int64_t steps = 0;
+    bool keep_on = false;
+    // per-row maxima over the layers (scratch sizing)
+    int64_t m_in = 0, m_hr = 0, m_hv = 0, m_gu = 0, m_act = 0, m_top = 0, m_e = 0;
+};
+
+static inline float bf16_to_float(uint16_t h) {
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+static inline uint16_t float_to_bf16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+static float host_elem(const HostTensor& t, int64_t i) {
+    if (t.dtype == 0) return bf16_to_float(((const uint16_t*)t.data.data())[i]);
+    if (t.dtype == 2) return ((const float*)t.data.data())[i];
+    return (float)((const int32_t*)t.data.data())[i];
+}
+
+static int lm_alloc(LayeredModel* m, void** p, size_t bytes) {
+    QIE_TRY(dmalloc(p, bytes));
+    m->allocs.push_back(*p);
+    return 0;
+}
+
+static const HostTensor* lm_find(LayeredModel* m, const std::string& name, std::initializer_list<int64_t> shape) {
+    auto it = m->host.find(name);
+    if (it == m->host.end()) {
+        fail(-22, "layered weights: tensor '%s' is missing", name.c_str());
+        return nullptr;
+    }
+    const HostTensor& t = it->second;
+    std::vector<int64_t> want(shape);
+    if (t.shape != want) {
+        std::string got, exp;
+        for (int64_t s : t.shape) got += std::to_string(s) + " ";
+        for (int64_t s : want) exp += std::to_string(s) + " ";
+        fail(-22, "layered weights: tensor '%s' has shape [%s], the architecture needs [%s]", name.c_str(), got.c_str(),
+             exp.c_str());
+        return nullptr;
+    }
+    if (t.dtype == 1) {
+        fail(-22, "layered weights: tensor '%s' is an integer table", name.c_str());
+        return nullptr;
+    }
+    return &t;
+}
+
+// rows [r0, r0 + t.rows) of a device matrix of `cols` columns in the model's weight type
+static int lm_upload_rows(LayeredModel* m, void* dev, int64_t r0, int64_t cols, const HostTensor& t,
+                          const std::vector<int64_t>* perm = nullptr) {
+    const int64_t n = t.numel();
+    char* dst = (char*)dev + (size_t)r0 * cols * m->esz();
+    if (m->f32) {
+        std::vector<float> tmp(n);
+        for (int64_t i = 0; i < n; i++) tmp[i] = host_elem(t, perm ? (*perm)[i] : i);
+        QIE_HIP(hipMemcpy(dst, tmp.data(), (size_t)n * 4, hipMemcpyHostToDevice));
+    } else {
+        std::vector<uint16_t> tmp(n);
+        for (int64_t i = 0; i < n; i++) {
+            const int64_t s = perm ? (*perm)[i] : i;
+            tmp[i] = t.dtype == 0 ? ((const uint16_t*)t.data.data())[s] : float_to_bf16(host_elem(t, s));
+        }
+        QIE_HIP(hipMemcpy(dst, tmp.data(), (size_t)n * 2, hipMemcpyHostToDevice));
+    }
+    return 0;
+}
+
+static int lm_floats(LayeredModel* m, float** dev, const HostTensor& t) {
+    const int64_t n = t.numel();
+    std::vector<float> tmp(n);
+    for (int64_t i = 0; i < n; i++) tmp[i] = host_elem(t, i);
+    QIE_TRY(lm_alloc(m, (void**)dev, (size_t)n * 4));
+    QIE_HIP(hipMemcpy(*dev, tmp.data(), (size_t)n * 4, hipMemcpyHostToDevice));
+    return 0;
+}
+
+static int lm_rope(LayeredModel* m, qie_engine* e, double base, int dims, int* index) {
+    for (size_t i = 0; i < m->ropes.size(); i++)
+        if (m->ropes[i].base == base && m->ropes[i].dims == dims) {
+            *index = (int)i;
+            return 0;
+        }
+    const int half = dims / 2, rows = e->opts.max_ctx;
+    std::vector<float> cs((size_t)rows * half), sn((size_t)rows * half);
+    for (int j = 0; j < half; j++) {
+        const double f = std::pow(base, -2.0 * j / dims);
+        for (int p = 0; p < rows; p++) {
+            cs[(size_t)p * half + j] = (float)std::cos(p * f);
+            sn[(size_t)p * half + j] = (float)std::sin(p * f);
+        }
+    }
+    RopeTab t{base, dims, nullptr, nullptr};
+    QIE_TRY(lm_alloc(m, (void**)&t.cs, cs.size() * 4 + 16));
+    QIE_TRY(lm_alloc(m, (void**)&t.sn, sn.size() * 4 + 16));
+    QIE_HIP(hipMemcpy(t.cs, cs.data(), cs.size() * 4, hipMemcpyHostToDevice));
+    QIE_HIP(hipMemcpy(t.sn, sn.data(), sn.size() * 4, hipMemcpyHostToDevice));
+    *index = (int)m->ropes.size();
+    m->ropes.push_back(t);
+    return 0;
+}
+
+void layered_engine_destroy(qie_engine* e) {
+    if (!e || !e->lm) return;
+    for (void* p : e->lm->allocs) hipFree(p);
+    delete e->lm;
+    e->lm = nullptr;
+}
+
+#define LM_GET(var, name, ...)                                   \
+    const HostTensor* var = lm_find(m, name, {__VA_ARGS__});     \
+    if (!var) return -22
+
+static int finalize_layer(qie_engine* e, LayeredModel* m, int i) {
+    LayerDev& L = m->L[i];
+    const qie_layer_desc& d = L.d;
+    const int64_t W = m->a.width, H = d.heads, hq = d.dim + d.rot_dim, R = d.kv_rank;
+    const std::string pl = "l" + std::to_string(i) + ".", px = pl + "mix.";
+    const bool own = d.kv_from < 0;
+    LM_GET(tq, px + "q", H * hq, W);
+    LM_GET(tg, px + "g", H, W);
+    const int64_t n_kv = own ? R + d.rot_dim : 0;
+    L.n_in = (int)(H * hq + n_kv + H);
+    L.g_col = (int)(H * hq + n_kv);
+    QIE_TRY(lm_alloc(m, &L.w_in, (size_t)L.n_in * W * m->esz()));
+    QIE_TRY(lm_upload_rows(m, L.w_in, 0, W, *tq));
+    if (own) {
+        LM_GET(tk, px + "dkv", R + d.rot_dim, W);
+        LM_GET(tn, px + "dkv.norm", R);
+        QIE_TRY(lm_upload_rows(m, L.w_in, H * hq, W, *tk));
+        QIE_TRY(lm_floats(m, &L.dkv_norm, *tn));
+    }
+    QIE_TRY(lm_upload_rows(m, L.w_in, L.g_col, W, *tg));
+    LM_GET(tuk, px + "uk", H * d.dim, R);
+    {   // [heads][dim][R] -> [heads][R][dim]: the absorbed query is q_nope W_uk,h, a product over dim
+        std::vector<int64_t> perm((size_t)H * d.dim * R);
+        for (int64_t h = 0; h < H; h++)
+            for (int64_t r = 0; r < R; r++)
+                for (int64_t k = 0; k < d.dim; k++) perm[(h * R + r) * d.dim + k] = (h * d.dim + k) * R + r;
+        QIE_TRY(lm_alloc(m, &L.uk_t, perm.size() * m->esz()));
+        QIE_TRY(lm_upload_rows(m, L.uk_t, 0, d.dim, *tuk, &perm));
+    }
+    LM_GET(tuv, px + "uv", H * d.vdim, R);
+    QIE_TRY(lm_alloc(m, &L.uv, (size_t)tuv->numel() * m->esz()));
+    QIE_TRY(lm_upload_rows(m, L.uv, 0, R, *tuv));
+    LM_GET(to, px + "o", W, H * d.vdim);
+    QIE_TRY(lm_alloc(m, &L.wo, (size_t)to->numel() * m->esz()));
+    QIE_TRY(lm_upload_rows(m, L.wo, 0, H * d.vdim, *to));
+    LM_GET(n1, pl + "norm1");
+    L.g1 = host_elem(*n1, 0);
+    QIE_TRY(lm_rope(m, e, (double)d.rot_base, d.rot_dims, &L.rope));
+    if (d.ff_kind != QIE_FF_NONE) {
+        LM_GET(n2, pl + "norm2");
+        L.g2 = host_elem(*n2, 0);
+    }
+    const int64_t ff = d.ff;
+    if (d.ff_kind == QIE_FF_DENSE) {
+        LM_GET(wg, pl + "mlp.gate", ff, W);
+        LM_GET(wu, pl + "mlp.up", ff, W);
+        LM_GET(wd, pl + "mlp.down", W, ff);
+        QIE_TRY(lm_alloc(m, &L.w_gu, (size_t)2 * ff * W * m->esz()));
+        QIE_TRY(lm_upload_rows(m, L.w_gu, 0, W, *wg));
+        QIE_TRY(lm_upload_rows(m, L.w_gu, ff, W, *wu));
+        QIE_TRY(lm_alloc(m, &L.w_down, (size_t)W * ff * m->esz()));
+        QIE_TRY(lm_upload_rows(m, L.w_down, 0, ff, *wd));
+    } else if (d.ff_kind == QIE_FF_MOE) {
+        const int64_t E = d.experts;
+        LM_GET(wr, pl + "mlp.router", E, W);
+        QIE_TRY(lm_alloc(m, &L.w_router, (size_t)E * W * m->esz()));
+        QIE_TRY(lm_upload_rows(m, L.w_router, 0, W, *wr));
+        QIE_TRY(lm_alloc(m, &L.w_gu, (size_t)E * 2 * ff * W * m->esz()));
+        QIE_TRY(lm_alloc(m, &L.w_down, (size_t)E * W * ff * m->esz()));
+        for (int64_t x = 0; x < E; x++) {
+            const std::string pe = pl + "mlp.e" + std::to_string(x) + ".";
+            LM_GET(wg, pe + "gate", ff, W);
+            LM_GET(wu, pe + "up", ff, W);
+            LM_GET(wd, pe + "down", W, ff);
+            QIE_TRY(lm_upload_rows(m, L.w_gu, x * 2 * ff, W, *wg));
+            QIE_TRY(lm_upload_rows(m, L.w_gu, x * 2 * ff + ff, W, *wu));
+            QIE_TRY(lm_upload_rows(m, L.w_down, x * W, ff, *wd));
+        }
+    }
+    if (m->a.depth_mix) {
+        LM_GET(da, pl + "dwa", (int64_t)i + 2);
+        QIE_TRY(lm_floats(m, &L.dwa, *da));
+    }
+    return 0;
+}
+
+// ------------------------------------------------------------------ the step
+static int lin(const qie_engine* e, const float* A, int64_t lda, const void* Wt, int64_t ldw, float* Y, int64_t ldy, int M, int N,
+               int K, int batch = 1, int64_t sA = 0, int64_t sW = 0, int64_t sY = 0, const int32_t* grp = nullptr) {
+    lay::LinearP p{A, lda, Wt, ldw, Y, ldy, M, N, K, batch, sA, sW, sY, e->lm->f32 ? 0 : 1, grp};
+    return lay::linear(p, e->lm->f32, e->stream);
+}
+
+static lay::LatentCache cache_of(const qie_batch* b) {
+    return lay::LatentCache{b->kc, b->seq_stride, b->d_table, b->page_tokens, b->max_pages};
+}
+
+static int enq_input_proj(qie_batch* b, int i, const float* xin, int T) {
+    const qie_engine* e = b->e;
+    const LayeredModel* m = e->lm;
+    const LayerDev& L = m->L[i];
+    LayeredBatch* s = b->lb;
+    return lin(e, xin, m->a.width, L.w_in, m->a.width, s->proj, L.n_in, T, L.n_in, m->a.width);
+}
+
+static int enq_latent_post(qie_batch* b, int i, int T) {
+    const qie_engine* e = b->e;
+    const LayeredModel* m = e->lm;
+    const LayerDev& L = m->L[i];
+    const qie_layer_desc& d = L.d;
+    LayeredBatch* s = b->lb;
+    lay::LatentPostP p{};
+    p.proj = s->proj;
+    p.ld = L.n_in;
+    p.row_slot = s->row_slot;
+    p.row_pos = s->row_pos;
+    p.heads = d.heads; p.dim = d.dim; p.rot = d.rot_dim; p.rot_dims = d.rot_dims; p.R = d.kv_rank;
+    p.own_kv = d.kv_from < 0;
+    p.norm_w = L.dkv_norm;
+    p.eps = m->a.norm_eps;
+    p.rope_cos = m->ropes[L.rope].cs;
+    p.rope_sin = m->ropes[L.rope].sn;
+    p.cache = cache_of(b);
+    p.layer_off = s->layer_off[L.cache_layer];
+    return lay::latent_post(p, m->f32, T, e->stream);
+}
+
+static int enq_absorb(qie_batch* b, int i, int T) {
+    const qie_engine* e = b->e;
+    const LayerDev& L = e->lm->L[i];
+    const qie_layer_desc& d = L.d;
+    LayeredBatch* s = b->lb;
+    const int hq = d.dim + d.rot_dim;
+    return lin(e, s->proj, L.n_in, L.uk_t, d.dim, s->qabs, (int64_t)d.heads * d.kv_rank, T, d.kv_rank, d.dim, d.heads, hq,
+               (int64_t)d.kv_rank * d.dim, d.kv_rank);
+}
+
+static int enq_attention(qie_batch* b, int i, int T) {
+    const qie_engine* e = b->e;
+    const LayeredModel* m = e->lm;
+    const LayerDev& L = m->L[i];
+    const qie_layer_desc& d = L.d;
+    LayeredBatch* s = b->lb;
+    lay::LatentAttnP p{};
+    p.q_abs = s->qabs;
+    p.proj = s->proj;
+    p.ld = L.n_in;
+    p.row_slot = s->row_slot;
+    p.row_pos = s->row_pos;
+    p.heads = d.heads; p.dim = d.dim; p.rot = d.rot_dim; p.R = d.kv_rank; p.window = d.window;
+    p.scale = d.scale;
+    p.cache = cache_of(b);
+    p.layer_off = s->layer_off[L.cache_layer];
+    p.out = s->olat;
+    return lay::latent_attention(p, m->f32, T, e->stream);
+}
+
+static int enq_mixer_out(qie_batch* b, int i, int T) {
+    const qie_engine* e = b->e;
+    const LayeredModel* m = e->lm;
+    const LayerDev& L = m->L[i];
+    const qie_layer_desc& d = L.d;
+    LayeredBatch* s = b->lb;
+    const int64_t HV = (int64_t)d.heads * d.vdim;
+    QIE_TRY(lin(e, s->olat, (int64_t)d.heads * d.kv_rank, L.uv, d.kv_rank, s->ov, HV, T, d.vdim, d.kv_rank, d.heads, d.kv_rank,
+                (int64_t)d.vdim * d.kv_rank, d.vdim));
+    QIE_TRY(lay::head_gate(s->ov, s->proj, L.n_in, L.g_col, d.heads, d.vdim, T, e->stream));
+    return lin(e, s->ov, HV, L.wo, HV, s->mix, m->a.width, T, m->a.width, (int)HV);
+}
+
+// feed-forward of layer i on rows y -> ffo
+static int enq_ff(qie_batch* b, int i, int T) {
+    const qie_engine* e = b->e;
+    const LayeredModel* m = e->lm;
+    const LayerDev& L = m->L[i];
+    const qie_layer_desc& d = L.d;
+    LayeredBatch* s = b->lb;
+    const int W = m->a.width, ff = d.ff;
+    hipStream_t st = e->stream;
+    if (d.ff_kind == QIE_FF_DENSE) {
+        QIE_TRY(lin(e, s->y, W, L.w_gu, W, s->gu, 2 * ff, T, 2 * ff, W));
+        QIE_TRY(lay::silu_mul(s->gu, s->act, T, ff, st));
+        return lin(e, s->act, ff, L.w_down, ff, s->ffo, W, T, W, ff);
+    }
+    const int E = d.experts, top = d.top, n = T * top;
+    QIE_TRY(lay::route_sigmoid_topk(s->y, L.w_router, m->f32, T, W, E, top, s->sel, s->score, st));
+    QIE_TRY(lay::moe_group(s->sel, n, E, s->cnt, s->off, s->slot_of, st));
+    QIE_TRY(lay::moe_gather(s->y, s->score, s->slot_of, T, top, W, s->xg, st));
+    QIE_TRY(lin(e, s->xg, W, L.w_gu, W, s->gu, 2 * ff, n, 2 * ff, W, E, 0, (int64_t)2 * ff * W, 0, s->off));
+    QIE_TRY(lay::silu_mul(s->gu, s->act, n, ff, st));
+    QIE_TRY(lin(e, s->act, ff, L.w_down, ff, s->yd, W, n, W, ff, E, 0, (int64_t)W * ff, 0, s->off));
+    return lay::moe_combine(s->yd, s->slot_of, T, top, W, s->ffo, st);
+}
+
+static int enq_layer(qie_batch* b, int i, const float* xin, int T, const float** xout) {
+    const qie_engine* e = b->e;
+    const LayeredModel* m = e->lm;
+    const LayerDev& L = m->L[i];
+    LayeredBatch* s = b->lb;
+    const int W = m->a.width;
+    hipStream_t st = e->stream;
+    const int64_t plane = s->cap * W;
+    float* result = s->stack + (int64_t)(i + 1) * plane;
+    QIE_TRY(enq_input_proj(b, i, xin, T));
+    QIE_TRY(enq_latent_post(b, i, T));
+    QIE_TRY(enq_absorb(b, i, T));
+    QIE_TRY(enq_attention(b, i, T));
+    QIE_TRY(enq_mixer_out(b, i, T));
+    const bool has_ff = L.d.ff_kind != QIE_FF_NONE;
+    QIE_TRY(lay::postnorm_add(xin, s->mix, has_ff ? s->y : result, T, W, L.g1, m->a.norm_eps, st));
+    if (has_ff) {
+        QIE_TRY(enq_ff(b, i, T));
+        QIE_TRY(lay::postnorm_add(s->y, s->ffo, result, T, W, L.g2, m->a.norm_eps, st));
+    }
+    if (m->a.depth_mix) {
+        QIE_TRY(lay::depth_mix(s->stack, plane, L.dwa, i + 2, s->x, (int64_t)T * W, st));
+        *xout = s->x;
+    } else {
+        *xout = result;
+    }
+    if (s->keep_on && s->keep)
+        QIE_HIP(hipMemcpyAsync(s->keep + (int64_t)i * plane, *xout, (size_t)T * W * 4, hipMemcpyDeviceToDevice, st));
+    return 0;
+}
+
+static int enq_forward(qie_batch* b, int T, int n_want) {
+    const qie_engine* e = b->e;
+    const LayeredModel* m = e->lm;
+    LayeredBatch* s = b->lb;
+    const int W = m->a.width;
+    QIE_TRY(lay::embed_rows(m->embed, m->f32, s->tok, s->stack, T, W, m->a.vocab, e->stream));
+    const float* x = s->stack;
+    for (int i = 0; i < m->a.n_layers; i++) QIE_TRY(enq_layer(b, i, x, T, &x));
+    if (n_want > 0) {
+        QIE_TRY(lay::final_rows(x, s->want, s->xn, n_want, W, m->g_final, m->a.norm_eps, e->stream));
+        QIE_TRY(lin(e, s->xn, W, m->head, W, s->logits, m->a.vocab, n_want, m->a.vocab, W));
+    }
+    return 0;
+}
+
+static void lb_free(LayeredBatch* s) {
+    void* ps[] = {s->stack, s->x, s->proj, s->qabs, s->olat, s->ov, s->mix, s->y, s->gu, s->act, s->ffo, s->xg, s->yd, s->score,
+                  s->row_slot, s->row_pos, s->tok, s->sel, s->cnt, s->off, s->slot_of, s->keep};
+    for (void* p : ps)
+        if (p) hipFree(p);
+    s->stack = s->x = s->proj = s->qabs = s->olat = s->ov = s->mix = s->y = s->gu = s->act = s->ffo = s->xg = s->yd = s->score =
+        s->keep = nullptr;
+    s->row_slot = s->row_pos = s->tok = s->sel = s->cnt = s->off = s->slot_of = nullptr;
+    s->cap = 0;
+}
+
+static int ensure_rows(qie_batch* b, int64_t T) {
+    LayeredBatch* s = b->lb;
+    const LayeredModel* m = b->e->lm;
+    if (T > s->cap) {
+        QIE_HIP(hipStreamSynchronize(b->e->stream));
+        lb_free(s);
+        const int64_t cap = (T + 63) / 64 * 64, W = m->a.width, L = m->a.n_layers;
+        int rc = 0;
+        auto A = [&](void** p, int64_t elems, size_t sz = 4) {
+            if (!rc) rc = dmalloc(p, (size_t)elems * sz);
+        };
+        A((void**)&s->stack, (L + 1) * cap * W);
+        A((void**)&s->x, cap * W);
+        A((void**)&s->proj, cap * s->m_in);
+        A((void**)&s->qabs, cap * s->m_hr);
+        A((void**)&s->olat, cap * s->m_hr);
+        A((void**)&s->ov, cap * s->m_hv);
+        A((void**)&s->mix, cap * W);
+        A((void**)&s->y, cap * W);
+        A((void**)&s->gu, cap * std::max<int64_t>(s->m_gu, 1));
+        A((void**)&s->act, cap * std::max<int64_t>(s->m_act, 1));
+        A((void**)&s->ffo, cap * W);
+        A((void**)&s->xg, cap * std::max<int64_t>(s->m_top, 1) * W);
+        A((void**)&s->yd, cap * std::max<int64_t>(s->m_top, 1) * W);
+        A((void**)&s->score, cap * std::max<int64_t>(s->m_top, 1));
+        A((void**)&s->sel, cap * std::max<int64_t>(s->m_top, 1));
+        A((void**)&s->slot_of, cap * std::max<int64_t>(s->m_top, 1));
+        A((void**)&s->cnt, s->m_e + 1);
+        A((void**)&s->off, s->m_e + 2);
+        A((void**)&s->row_slot, cap);
+        A((void**)&s->row_pos, cap);
+        A((void**)&s->tok, cap);
+        if (s->keep_on) A((void**)&s->keep, L * cap * W);
+        if (rc) return rc;
+        s->cap = cap;
+    }
+    if (s->keep_on && !s->keep) QIE_TRY(dmalloc((void**)&s->keep, (size_t)m->a.n_layers * s->cap * m->a.width * 4));
+    if (T > s->h_stage_rows) {
+        if (s->h_stage) hipHostFree(s->h_stage);
+        s->h_stage = nullptr;
+        const int64_t rows = (T + 255) / 256 * 256;
+        QIE_HIP(hipHostMalloc((void**)&s->h_stage, (size_t)rows * 3 * 4, hipHostMallocDefault));
+        s->h_stage_rows = rows;
+    }
+    return 0;
+}
+
+static int ensure_want(qie_batch* b, int64_t n) {
+    LayeredBatch* s = b->lb;
+    const LayeredModel* m = b->e->lm;
+    if (n <= s->want_cap) return 0;
+    QIE_HIP(hipStreamSynchronize(b->e->stream));
+    void* ps[] = {s->want, s->xn, s->logits, s->logits_bf, s->d_ids, s->d_step};
+    for (void* p : ps)
+        if (p) hipFree(p);
+    s->want = nullptr; s->xn = nullptr; s->logits = nullptr; s->logits_bf = nullptr; s->d_ids = nullptr; s->d_step = nullptr;
+    s->want_cap = 0;
+    const int64_t cap = (n + 15) / 16 * 16, V = m->a.vocab;
+    QIE_TRY(dmalloc((void**)&s->want, cap * 4));
+    QIE_TRY(dmalloc((void**)&s->xn, cap * m->a.width * 4));
+    QIE_TRY(dmalloc((void**)&s->logits, cap * V * 4));
+    QIE_TRY(dmalloc((void**)&s->logits_bf, cap * V * 2));
+    QIE_TRY(dmalloc((void**)&s->d_ids, cap * 4));
+    QIE_TRY(dmalloc((void**)&s->d_step, cap * 4));
+    if (b->samp_ws) hipFree(b->samp_ws);
+    b->samp_ws = nullptr;
+    QIE_TRY(dmalloc(&b->samp_ws, (size_t)qie_sample_workspace_bytes(cap, V)));
+    s->want_cap = cap;
+    return 0;
+}
+
+int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t page_tokens, int32_t n_pages, qie_batch** out) {
+    LayeredModel* m = e->lm;
+    QIE_REQUIRE(m->final, "qie_batch_create_paged: the layered engine's weights are not finalized");
+    QIE_REQUIRE(out && batch > 0 && batch <= 4096 && max_ctx > 1, "qie_batch_create_paged: bad arguments");
+    QIE_REQUIRE(max_ctx <= e->opts.max_ctx, "qie_batch_create_paged: max_ctx %d > engine max_ctx %d", max_ctx, e->opts.max_ctx);
+    if (page_tokens == 0) page_tokens = 64;
+    QIE_REQUIRE(page_tokens >= 16 && (page_tokens & (page_tokens - 1)) == 0,
+                "qie_batch_create_paged: page_tokens %d must be a power of two >= 16 (layered engines)", page_tokens);
+    QIE_REQUIRE(n_pages == 0 || n_pages >= 2, "qie_batch_create_paged: need the scratch page and one more");
+    qie_batch* b = new qie_batch();
+    LayeredBatch* s = new LayeredBatch();
+    b->e = e;
+    b->lb = s;
+    b->B = batch;
+    b->max_ctx = max_ctx;
+    b->page_tokens = page_tokens;
+    b->max_pages = (max_ctx + page_tokens - 1) / page_tokens;
+    b->n_pages = n_pages > 0 ? n_pages : batch * b->max_pages + 1;
+    s->layer_off.assign(m->a.n_layers, 0);
+    int64_t off = 0;
+    for (int i = 0; i < m->a.n_layers; i++) {
+        const qie_layer_desc& d = m->L[i].d;
+        if (d.kv_from < 0) {
+            s->layer_off[i] = off;
+            off += (int64_t)page_tokens * (d.kv_rank + d.rot_dim);
+        }
+        const int64_t H = d.heads;
+        s->m_in = std::max<int64_t>(s->m_in, m->L[i].n_in);
+        s->m_hr = std::max<int64_t>(s->m_hr, H * d.kv_rank);
+        s->m_hv = std::max<int64_t>(s->m_hv, H * d.vdim);
+        const int64_t k = d.ff_kind == QIE_FF_MOE ? d.top : 1;
+        if (d.ff_kind != QIE_FF_NONE) {
+            s->m_gu = std::max<int64_t>(s->m_gu, k * 2 * d.ff);
+            s->m_act = std::max<int64_t>(s->m_act, k * d.ff);
+        }
+        if (d.ff_kind == QIE_FF_MOE) {
+            s->m_top = std::max<int64_t>(s->m_top, d.top);
+            s->m_e = std::max<int64_t>(s->m_e, d.experts);
+        }
+    }
+    b->seq_stride = off;   // elements per page
+    b->h_table.assign((size_t)batch * b->max_pages, 0);
+    for (int p = b->n_pages - 1; p >= 1; p--) b->free_pages.push_back(p);
+    b->held.assign(batch, 0);
+    b->idle.assign(batch, 1);
+    b->h_pos.assign(batch, 0);
+    b->table_dirty = true;
+    const size_t pool = (size_t)b->n_pages * off * m->esz();
+    int rc = dmalloc((void**)&b->kc, pool);
+    if (!rc) rc = dmalloc((void**)&b->d_table, b->h_table.size() * 4);
+    if (!rc) {
+        hipError_t he = hipMemsetAsync(b->kc, 0, pool, e->stream);
+        if (he == hipSuccess) he = hipStreamSynchronize(e->stream);
+        if (he != hipSuccess) rc = fail((int)he, "batch init: %s", hipGetErrorString(he));
+    }
+    if (!rc) rc = flush_table(b);
+    if (rc) {
+        qie_batch_destroy(b);
+        return rc;
+    }
+    *out = b;
+    return 0;
+}
+
+void layered_batch_destroy(qie_batch* b) {
+    LayeredBatch* s = b->lb;
+    if (!s) return;
+    lb_free(s);
+    void* ps[] = {s->want, s->xn, s->logits, s->logits_bf, s->d_ids, s->d_step};
+    for (void* p : ps)
+        if (p) hipFree(p);
+    if (s->h_stage) hipHostFree(s->h_stage);
+    delete s;
+    b->lb = nullptr;
+}
+
+}  // namespace qie
+
+using namespace qie;
+
+extern "C" {
+
+int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* opts, qie_engine** out) {
+    QIE_REQUIRE(arch && out && arch->layers, "qie_engine_create_layered: bad arguments");
+    QIE_REQUIRE(arch->n_layers > 0 && arch->width > 0 && arch->vocab > 0 && arch->norm_eps >= 0.f,
+                "qie_engine_create_layered: invalid sizes");
+    QIE_REQUIRE(!opts || !opts->tp_comm, "qie_engine_create_layered: layered engines run on one device");
+    QIE_REQUIRE(!opts || (!opts->weight_fp8 && !opts->prefill_fp8), "qie_engine_create_layered: fp8 weights are not covered");
+    for (int i = 0; i < arch->n_layers; i++) {
+        const qie_layer_desc& d = arch->layers[i];
+        QIE_REQUIRE(d.mixer == QIE_MIXER_LATENT_ATTENTION, "layer %d: unknown mixer %d", i, d.mixer);
+        QIE_REQUIRE(d.heads > 0 && d.dim > 0 && d.rot_dim >= 0 && d.vdim > 0 && d.kv_rank > 0 && d.window > 0,
+                    "layer %d: invalid mixer sizes", i);
+        QIE_REQUIRE(d.rot_dims >= 0 && d.rot_dims % 2 == 0 && d.rot_dims <= d.rot_dim, "layer %d: rotary dims %d of %d", i,
+                    d.rot_dims, d.rot_dim);
+        QIE_REQUIRE(d.rot_dims == 0 || d.rot_base > 0.f, "layer %d: rotary base", i);
+        if (d.kv_from >= 0) {
+            QIE_REQUIRE(d.kv_from < i, "layer %d: kv_from %d must name an earlier layer", i, d.kv_from);
+            const qie_layer_desc& o = arch->layers[d.kv_from];
+            QIE_REQUIRE(o.kv_from < 0 && o.kv_rank == d.kv_rank && o.rot_dim == d.rot_dim && o.rot_dims == d.rot_dims &&
+                            o.rot_base == d.rot_base,
+                        "layer %d: the layer it reads its cache from (%d) must own one of the same shape and rotation", i,
+                        d.kv_from);
+        }
+        QIE_REQUIRE(d.ff_kind >= QIE_FF_NONE && d.ff_kind <= QIE_FF_MOE, "layer %d: unknown feed-forward %d", i, d.ff_kind);
+        QIE_REQUIRE(d.ff_kind == QIE_FF_NONE || d.ff > 0, "layer %d: feed-forward size", i);
+        QIE_REQUIRE(d.ff_kind != QIE_FF_MOE || (d.experts > 0 && d.top > 0 && d.top <= d.experts), "layer %d: %d of %d experts", i,
+                    d.top, d.experts);
+    }
+    qie_engine* e = new qie_engine();
+    if (opts) e->opts = *opts;
+    if (e->opts.max_ctx <= 0) e->opts.max_ctx = 4096;
+    e->opts.use_graph = 0;
+    e->opts.tp_size = 1;
+    e->opts.tp_rank = 0;
+    e->sh.tp = 1;
+    LayeredModel* m = new LayeredModel();
+    e->lm = m;
+    m->a = *arch;
+    m->descs.assign(arch->layers, arch->layers + arch->n_layers);
+    m->a.layers = m->descs.data();
+    m->f32 = e->opts.compute_f32 != 0;
+    m->L.resize(arch->n_layers);
+    for (int i = 0; i < arch->n_layers; i++) {
+        m->L[i].d = m->descs[i];
+        m->L[i].cache_layer = m->descs[i].kv_from >= 0 ? m->descs[i].kv_from : i;
+    }
+    // informational mirror for qie_engine_spec
+    e->spec.n_layers = arch->n_layers;
+    e->spec.hidden = arch->width;
+    e->spec.vocab = arch->vocab;
+    e->spec.rms_eps = arch->norm_eps;
+    hipError_t he = hipSetDevice(e->opts.device);
+    if (he == hipSuccess) he = hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking);
+    if (he != hipSuccess) {
+        qie_engine_destroy(e);
+        return fail((int)he, "qie_engine_create_layered: %s", hipGetErrorString(he));
+    }
+    *out = e;
+    return 0;
+}
+
+int qie_engine_put_tensor(qie_engine* e, const char* name, const void* host, int32_t dtype, int32_t ndim, const int64_t* shape) {
+    QIE_REQUIRE(e && e->lm && name && host && dtype >= 0 && dtype <= 2 && ndim >= 0 && ndim <= 4 && (ndim == 0 || shape),
+                "qie_engine_put_tensor: bad arguments (layered engines)");
+    QIE_REQUIRE(!e->lm->final, "qie_engine_put_tensor: weights are finalized");
+    HostTensor t;
+    t.dtype = dtype;
+    t.shape.assign(shape, shape + ndim);
+    const int64_t n = t.numel();
+    QIE_REQUIRE(n >= 0, "qie_engine_put_tensor: bad shape");
+    t.data.resize((size_t)n * (dtype == 0 ? 2 : 4));
+    memcpy(t.data.data(), host, t.data.size());
+    e->lm->host[name] = std::move(t);
+    return 0;
+}
+
+int qie_engine_finalize_weights(qie_engine* e) {
+    QIE_REQUIRE(e && e->lm, "qie_engine_finalize_weights: a layered engine");
+    LayeredModel* m = e->lm;
+    QIE_REQUIRE(!m->final, "qie_engine_finalize_weights: already done");
+    QIE_HIP(hipSetDevice(e->opts.device));
+    const int64_t W = m->a.width, V = m->a.vocab;
+    LM_GET(te, "embed", V, W);
+    LM_GET(th, "head", V, W);
+    LM_GET(tn, "final.norm");
+    QIE_TRY(lm_alloc(m, &m->embed, (size_t)V * W * m->esz()));
+    QIE_TRY(lm_upload_rows(m, m->embed, 0, W, *te));
+    QIE_TRY(lm_alloc(m, &m->head, (size_t)V * W * m->esz()));
+    QIE_TRY(lm_upload_rows(m, m->head, 0, W, *th));
+    m->g_final = host_elem(*tn, 0);
+    for (int i = 0; i < m->a.n_layers; i++) QIE_TRY(finalize_layer(e, m, i));
+    m->host.clear();
+    m->final = true;
+    e->have_weights = true;
+    return 0;
+}
+
+int qie_batch_step(qie_batch* b, int32_t n_entries, const int32_t* slots, const int32_t* counts, const int32_t* tokens,
+                   int32_t n_want, const int32_t* want_rows, float* host_logits) {
+    QIE_REQUIRE(b && b->lb, "qie_batch_step: a batch of a layered engine");
+    QIE_REQUIRE(n_entries > 0 && slots && counts && tokens && n_want >= 0 && (n_want == 0 || want_rows),
+                "qie_batch_step: bad arguments");
+    qie_engine* e = b->e;
+    LayeredBatch* s = b->lb;
+    QIE_HIP(hipSetDevice(e->opts.device));
+    int64_t T = 0, new_pages = 0;
+    std::vector<char> seen(b->B, 0);
+    for (int i = 0; i < n_entries; i++) {
+        const int sl = slots[i];
+        QIE_REQUIRE(sl >= 0 && sl < b->B && !seen[sl], "qie_batch_step: entry %d: slot %d out of range or repeated", i, sl);
+        seen[sl] = 1;
+        QIE_REQUIRE(counts[i] > 0, "qie_batch_step: entry %d: empty", i);
+        const int64_t p0 = b->idle[sl] ? 0 : b->h_pos[sl], p1 = p0 + counts[i];
+        QIE_REQUIRE(p1 <= b->max_ctx, "qie_batch_step: slot %d would hold %lld tokens, max_ctx %d", sl, (long long)p1, b->max_ctx);
+        const int64_t held = b->idle[sl] ? 0 : b->held[sl];
+        new_pages += std::max<int64_t>(0, (p1 + b->page_tokens - 1) / b->page_tokens - held);
+        T += counts[i];
+    }
+    QIE_REQUIRE(new_pages <= (int64_t)b->free_pages.size(), "qie_batch_step: the step needs %lld more pages, %zu free",
+                (long long)new_pages, b->free_pages.size());
+    for (int i = 0; i < n_want; i++)
+        QIE_REQUIRE(want_rows[i] >= 0 && want_rows[i] < T, "qie_batch_step: wanted row %d outside the step's %lld rows",
+                    want_rows[i], (long long)T);
+    QIE_TRY(ensure_rows(b, T));
+    QIE_TRY(ensure_want(b, std::max(n_want, 1)));
+    int32_t* hs = s->h_stage;
+    const int64_t R = s->h_stage_rows;
+    int64_t r = 0;
+    for (int i = 0; i < n_entries; i++) {
+        const int sl = slots[i];
+        if (b->idle[sl]) {
+            b->idle[sl] = 0;
+            b->h_pos[sl] = 0;
+        }
+        QIE_TRY(ensure_pages(b, sl, (int64_t)b->h_pos[sl] + counts[i]));
+        for (int k = 0; k < counts[i]; k++, r++) {
+            hs[r] = sl;
+            hs[R + r] = b->h_pos[sl] + k;
+            hs[2 * R + r] = tokens[r];
+        }
+        b->h_pos[sl] += counts[i];
+    }
+    QIE_TRY(flush_table(b));
+    hipStream_t st = e->stream;
+    QIE_HIP(hipMemcpyAsync(s->row_slot, hs, (size_t)T * 4, hipMemcpyHostToDevice, st));
+    QIE_HIP(hipMemcpyAsync(s->row_pos, hs + R, (size_t)T * 4, hipMemcpyHostToDevice, st));
+    QIE_HIP(hipMemcpyAsync(s->tok, hs + 2 * R, (size_t)T * 4, hipMemcpyHostToDevice, st));
+    if (n_want > 0) QIE_HIP(hipMemcpyAsync(s->want, want_rows, (size_t)n_want * 4, hipMemcpyHostToDevice, st));
+    QIE_TRY(enq_forward(b, (int)T, n_want));
+    s->last_T = (int)T;
+    s->last_want = n_want;
+    s->steps++;
+    if (host_logits && n_want > 0)
+        QIE_HIP(hipMemcpyAsync(host_logits, s->logits, (size_t)n_want * e->lm->a.vocab * 4, hipMemcpyDeviceToHost, st));
+    // the staging rows and the caller's arrays are free again after this
+    QIE_HIP(hipStreamSynchronize(st));
+    return 0;
+}
+
+int qie_batch_step_sample(qie_batch* b, const qie_sampling* smp, int32_t* host_ids) {
+    QIE_REQUIRE(b && b->lb && smp && host_ids, "qie_batch_step_sample: bad arguments");
+    LayeredBatch* s = b->lb;
+    const int n = s->last_want;
+    QIE_REQUIRE(n > 0, "qie_batch_step_sample: the last step wanted no rows");
+    qie_engine* e = b->e;
+    hipStream_t st = e->stream;
+    const int64_t V = e->lm->a.vocab;
+    QIE_TRY(lay::rows_to_bf16(s->logits, s->logits_bf, (int64_t)n * V, st));
+    std::vector<int32_t> steps(n, (int32_t)(s->steps & 0x7fffffff));
+    QIE_HIP(hipMemcpyAsync(s->d_step, steps.data(), (size_t)n * 4, hipMemcpyHostToDevice, st));
+    QIE_HIP(hipStreamSynchronize(st));
+    QIE_TRY(qie_sample(s->logits_bf, n, V, V, smp, s->d_step, s->d_ids, b->samp_ws, st));
+    QIE_HIP(hipMemcpyAsync(host_ids, s->d_ids, (size_t)n * 4, hipMemcpyDeviceToHost, st));
+    QIE_HIP(hipStreamSynchronize(st));
+    return 0;
+}
+
+int qie_batch_keep_layers(qie_batch* b, int32_t enable) {
+    QIE_REQUIRE(b && b->lb, "qie_batch_keep_layers: a batch of a layered engine");
+    b->lb->keep_on = enable != 0;
+    return 0;
+}
+
+int qie_batch_step_layers(qie_batch* b, float* host_out, int64_t n) {
+    QIE_REQUIRE(b && b->lb && host_out, "qie_batch_step_layers: bad arguments");
+    LayeredBatch* s = b->lb;
+    const LayeredModel* m = b->e->lm;
+    const int64_t W = m->a.width, T = s->last_T, L = m->a.n_layers;
+    QIE_REQUIRE(s->keep && T > 0 && n >= L * T * W, "qie_batch_step_layers: nothing kept, or the buffer is too small");
+    QIE_HIP(hipStreamSynchronize(b->e->stream));
+    for (int64_t i = 0; i < L; i++)
+        QIE_HIP(hipMemcpy(host_out + i * T * W, s->keep + i * s->cap * W, (size_t)T * W * 4, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+int qie_batch_time_stage(qie_batch* b, int32_t which, int32_t layer, int32_t iters, double* avg_us) {
+    QIE_REQUIRE(b && b->lb && avg_us && iters > 0 && which >= 0 && which <= 3, "qie_batch_time_stage: bad arguments");
+    LayeredBatch* s = b->lb;
+    const LayeredModel* m = b->e->lm;
+    const int T = s->last_T;
+    QIE_REQUIRE(T > 0, "qie_batch_time_stage: run a step first");
+    QIE_REQUIRE(which == 0 || (layer >= 0 && layer < m->a.n_layers), "qie_batch_time_stage: layer %d", layer);
+    QIE_REQUIRE(which != 3 || m->L[layer].d.ff_kind != QIE_FF_NONE, "qie_batch_time_stage: layer %d has no feed-forward", layer);
+    hipStream_t st = b->e->stream;
+    hipEvent_t e0, e1;
+    QIE_HIP(hipEventCreate(&e0));
+    QIE_HIP(hipEventCreate(&e1));
+    int rc = 0;
+    auto once = [&]() -> int {
+        const float* xin = layer == 0 || which == 0 ? s->stack : s->x;
+        switch (which) {
+            case 0: return enq_forward(b, T, s->last_want);
+            case 1: return enq_attention(b, layer, T);
+            case 2:
+                QIE_TRY(enq_input_proj(b, layer, xin, T));
+                QIE_TRY(enq_absorb(b, layer, T));
+                return enq_mixer_out(b, layer, T);
+            default: return enq_ff(b, layer, T);
+        }
+    };
+    rc = once();   // warm
+    if (!rc) {
+        hipEventRecord(e0, st);
+        for (int i = 0; i < iters && !rc; i++) rc = once();
+        hipEventRecord(e1, st);
+        hipError_t he = hipEventSynchronize(e1);
+        float ms = 0.f;
+        if (he == hipSuccess) he = hipEventElapsedTime(&ms, e0, e1);
+        if (he != hipSuccess && !rc) rc = fail((int)he, "qie_batch_time_stage: %s", hipGetErrorString(he));
+        *avg_us = (double)ms * 1000.0 / iters;
+    }
+    hipEventDestroy(e0);
+    hipEventDestroy(e1);
+    return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,523 @@
+// k_layered.hip — kernels of the layered-model engine tier (engine_layered.hip): the
+// mechanisms that the Qwen decoder does not have, each with its constants as parameters.
+//
+//   lay::linear            y = A W^T, fp32 accumulation in k order; A fp32 (optionally rounded to
+//                          bf16 on load), W fp32 or bf16; batched (per head) and grouped (per
+//                          expert) forms
+//   lay::latent_post       latent KV: RMS norm of the compressed row, rotate-half rotary of the
+//                          shared key part and of every head's rotated query part, paged append
+//   lay::latent_attention  sliding-window attention over the latent cache in absorbed form
+//                          (scores against [c ; k_rot], output in latent space), online softmax
+//   lay::head_gate         per-head sigmoid output gate
+//   lay::postnorm_add      y = x + g * v / sqrt(mean(v^2) + eps): norm on the sublayer's output
+//   lay::depth_mix         x = sum_j a[j] X_j over the stack of earlier layer results
+//   lay::route_sigmoid_topk, moe_group, moe_gather, moe_combine: sigmoid router whose score
+//                          scales the expert's input, rows grouped by expert for the grouped linear
+//   lay::silu_mul, embed_rows, final_rows, rows_to_bf16
+//
+// Everything the residual stream, a norm, a router, a score or a softmax touches is fp32.  No
+// result depends on which other rows are in the launch: every output element is reduced in an
+// order fixed by its own sizes.
+#include "k_layered.hpp"
+
+namespace qie {
+namespace lay {
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p, int64_t i);
+template <> __device__ __forceinline__ float ldf<float>(const float* p, int64_t i) { return p[i]; }
+template <> __device__ __forceinline__ float ldf<uint16_t>(const uint16_t* p, int64_t i) { return bf2f(p[i]); }
+template <typename T> __device__ __forceinline__ void stf(T* p, int64_t i, float v);
+template <> __device__ __forceinline__ void stf<float>(float* p, int64_t i, float v) { p[i] = v; }
+template <> __device__ __forceinline__ void stf<uint16_t>(uint16_t* p, int64_t i, float v) { p[i] = f2bf(v); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+// block-wide sum over 256 threads (4 waves); every thread gets the result
+__device__ __forceinline__ float block_sum256(float v, float* red) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// ------------------------------------------------------------------ linear
+constexpr int LBM = 64, LBN = 64, LBK = 16;
+
+template <typename TW>
+__global__ __launch_bounds__(256) void linear_kernel(LinearP p) {
+    __shared__ float As[LBK][LBM + 4];
+    __shared__ float Ws[LBK][LBN + 4];
+    const int z = blockIdx.z;
+    int m_lo = 0, m_hi = p.M;
+    if (p.grp_off) {
+        m_lo = p.grp_off[z];
+        m_hi = p.grp_off[z + 1];
+    }
+    const int m0 = m_lo + blockIdx.y * LBM;
+    if (m0 >= m_hi) return;
+    const int n0 = blockIdx.x * LBN;
+    const float* A = p.A + (int64_t)z * p.sA;
+    const TW* W = (const TW*)p.W + (int64_t)z * p.sW;
+    float* Y = p.Y + (int64_t)z * p.sY;
+    const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < p.K; k0 += LBK) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int idx = tid + i * 256, r = idx >> 4, kk = idx & 15;
+            const int m = m0 + r, n = n0 + r, k = k0 + kk;
+            float a = 0.f, w = 0.f;
+            if (k < p.K) {
+                if (m < m_hi) {
+                    a = A[(int64_t)m * p.lda + k];
+                    if (p.round_a) a = rbf(a);
+                }
+                if (n < p.N) w = ldf<TW>(W, (int64_t)n * p.ldw + k);
+            }
+            As[kk][r] = a;
+            Ws[kk][r] = w;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < LBK; kk++) {
+            float a[4], w[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                a[i] = As[kk][ty * 4 + i];
+                w[i] = Ws[kk][tx * 4 + i];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= m_hi) continue;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int n = n0 + tx * 4 + j;
+            if (n < p.N) Y[(int64_t)m * p.ldy + n] = acc[i][j];
+        }
+    }
+}
+
+int linear(const LinearP& p, bool w_f32, hipStream_t st) {
+    QIE_REQUIRE(p.A && p.W && p.Y && p.M > 0 && p.N > 0 && p.K > 0 && p.batch > 0, "layered linear: bad arguments");
+    dim3 grid((unsigned)((p.N + LBN - 1) / LBN), (unsigned)((p.M + LBM - 1) / LBM), (unsigned)p.batch);
+    if (w_f32)
+        hipLaunchKernelGGL(linear_kernel<float>, grid, dim3(256), 0, st, p);
+    else
+        hipLaunchKernelGGL(linear_kernel<uint16_t>, grid, dim3(256), 0, st, p);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// ------------------------------------------------------------------ embedding rows
+template <typename TW>
+__global__ __launch_bounds__(256) void embed_rows_kernel(const TW* E, const int32_t* tok, float* out, int W, int vocab) {
+    const int t = blockIdx.x;
+    int id = tok[t];
+    if (id < 0 || id >= vocab) id = 0;
+    for (int w = threadIdx.x; w < W; w += 256) out[(int64_t)t * W + w] = ldf<TW>(E, (int64_t)id * W + w);
+}
+int embed_rows(const void* E, bool w_f32, const int32_t* tok, float* out, int T, int W, int vocab, hipStream_t st) {
+    if (w_f32)
+        hipLaunchKernelGGL(embed_rows_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)E, tok, out, W, vocab);
+    else
+        hipLaunchKernelGGL(embed_rows_kernel<uint16_t>, dim3(T), dim3(256), 0, st, (const uint16_t*)E, tok, out, W, vocab);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// ------------------------------------------------------------------ latent post-projection
+// One block per row.  proj row = [q (H x (dim + rot)) | c (R) | k_rot (rot) | ...].  The rotary
+// pairs coordinate i with i + dims/2 inside the first `dims` coordinates of a rotated part.
+__device__ __forceinline__ const void* latent_row(const LatentCache& c, int slot, int pos, int64_t layer_off, int D,
+                                                  int elem) {
+    const int page = c.table[(int64_t)slot * c.max_pages + pos / c.page_tokens];
+    const int64_t e = (int64_t)page * c.page_stride + layer_off + (int64_t)(pos % c.page_tokens) * D;
+    return (const char*)c.pool + e * elem;
+}
+
+template <typename TC>
+__global__ __launch_bounds__(256) void latent_post_kernel(LatentPostP p) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int slot = p.row_slot[t], pos = p.row_pos[t];
+    float* row = p.proj + (int64_t)t * p.ld;
+    const int half = p.rot_dims / 2;
+    const float* cs = p.rope_cos + (int64_t)pos * half;
+    const float* sn = p.rope_sin + (int64_t)pos * half;
+    const int hq = p.dim + p.rot;
+    // queries: rotate the rotated part of every head in place
+    for (int i = tid; i < p.heads * half; i += 256) {
+        const int h = i / half, j = i % half;
+        float* q = row + h * hq + p.dim;
+        const float u = q[j], v = q[j + half];
+        q[j] = u * cs[j] - v * sn[j];
+        q[j + half] = v * cs[j] + u * sn[j];
+    }
+    if (!p.own_kv) return;
+    const float* d = row + p.heads * hq;
+    float ss = 0.f;
+    for (int i = tid; i < p.R; i += 256) ss += d[i] * d[i];
+    ss = block_sum256(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)p.R + p.eps);
+    TC* out = (TC*)latent_row(p.cache, slot, pos, p.layer_off, p.R + p.rot, sizeof(TC));
+    for (int i = tid; i < p.R; i += 256) stf<TC>(out, i, d[i] * inv * p.norm_w[i]);
+    const float* kr = d + p.R;
+    for (int j = tid; j < p.rot; j += 256) {
+        float v;
+        if (j < half)
+            v = kr[j] * cs[j] - kr[j + half] * sn[j];
+        else if (j < p.rot_dims)
+            v = kr[j] * cs[j - half] + kr[j - half] * sn[j - half];
+        else
+            v = kr[j];
+        stf<TC>(out, p.R + j, v);
+    }
+}
+int latent_post(const LatentPostP& p, bool cache_f32, int T, hipStream_t st) {
+    QIE_REQUIRE(p.rot_dims % 2 == 0 && p.rot_dims <= p.rot, "latent_post: rotary dims %d must be even and <= %d", p.rot_dims,
+                p.rot);
+    if (cache_f32)
+        hipLaunchKernelGGL(latent_post_kernel<float>, dim3(T), dim3(256), 0, st, p);
+    else
+        hipLaunchKernelGGL(latent_post_kernel<uint16_t>, dim3(T), dim3(256), 0, st, p);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// ------------------------------------------------------------------ latent attention
+// One block per (head, row).  The query in latent space q' = [W_uk,h^T q_nope ; q_rot] (D = R +
+// rot floats) is scored against the cached rows [c_j ; k_rot_j] of positions
+// max(0, pos - window + 1) .. pos; the output is sum_j p_j c_j (R floats), expanded by W_uv
+// afterwards.  Keys go through in chunks of ATT_CHUNK with a running max and sum.
+constexpr int ATT_CHUNK = 256;
+constexpr int ATT_MAXR = 4;   // R <= 256 * ATT_MAXR
+
+template <typename TC>
+__global__ __launch_bounds__(256) void latent_attention_kernel(LatentAttnP p) {
+    extern __shared__ float sm[];
+    float* q = sm;                  // [D]
+    float* sc = sm + p.R + p.rot;   // [ATT_CHUNK]
+    __shared__ float red[4];
+    const int h = blockIdx.x, t = blockIdx.y, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int slot = p.row_slot[t], pos = p.row_pos[t];
+    const int D = p.R + p.rot;
+    const float* qa = p.q_abs + ((int64_t)t * p.heads + h) * p.R;
+    const float* qr = p.proj + (int64_t)t * p.ld + h * (p.dim + p.rot) + p.dim;
+    for (int i = tid; i < D; i += 256) q[i] = i < p.R ? qa[i] : qr[i - p.R];
+    __syncthreads();
+    int lo = pos - p.window + 1;
+    if (lo < 0) lo = 0;
+    float m_run = -INFINITY, l_run = 0.f;
+    float acc[ATT_MAXR] = {};
+    for (int j0 = lo; j0 <= pos; j0 += ATT_CHUNK) {
+        const int nk = min(ATT_CHUNK, pos + 1 - j0);
+        for (int jj = wave; jj < nk; jj += 4) {
+            const TC* k = (const TC*)latent_row(p.cache, slot, j0 + jj, p.layer_off, D, sizeof(TC));
+            float s = 0.f;
+            for (int i = lane; i < D; i += 64) s = fmaf(q[i], ldf<TC>(k, i), s);
+            s = wave_sum(s);
+            if (lane == 0) sc[jj] = s * p.scale;
+        }
+        __syncthreads();
+        float mx = -INFINITY;
+        for (int jj = tid; jj < nk; jj += 256) mx = fmaxf(mx, sc[jj]);
+        mx = wave_max(mx);
+        if (lane == 0) red[wave] = mx;
+        __syncthreads();
+        mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = expf(m_run - m_new);   // 0 on the first chunk
+        __syncthreads();
+        float ls = 0.f;
+        for (int jj = tid; jj < nk; jj += 256) {
+            const float e = expf(sc[jj] - m_new);
+            sc[jj] = e;
+            ls += e;
+        }
+        ls = block_sum256(ls, red);
+        l_run = l_run * alpha + ls;
+        m_run = m_new;
+#pragma unroll
+        for (int i = 0; i < ATT_MAXR; i++) acc[i] *= alpha;
+        for (int jj = 0; jj < nk; jj++) {
+            const TC* c = (const TC*)latent_row(p.cache, slot, j0 + jj, p.layer_off, D, sizeof(TC));
+            const float w = sc[jj];
+#pragma unroll
+            for (int i = 0; i < ATT_MAXR; i++) {
+                const int r = tid + i * 256;
+                if (r < p.R) acc[i] = fmaf(w, ldf<TC>(c, r), acc[i]);
+            }
+        }
+        __syncthreads();
+    }
+    const float inv = 1.0f / l_run;
+    float* o = p.out + ((int64_t)t * p.heads + h) * p.R;
+#pragma unroll
+    for (int i = 0; i < ATT_MAXR; i++) {
+        const int r = tid + i * 256;
+        if (r < p.R) o[r] = acc[i] * inv;
+    }
+}
+int latent_attention(const LatentAttnP& p, bool cache_f32, int T, hipStream_t st) {
+    QIE_REQUIRE(p.R <= 256 * ATT_MAXR, "latent attention: latent size %d above %d", p.R, 256 * ATT_MAXR);
+    QIE_REQUIRE(p.window >= 1, "latent attention: window %d", p.window);
+    const size_t shm = (size_t)(p.R + p.rot + ATT_CHUNK) * 4;
+    if (cache_f32)
+        hipLaunchKernelGGL(latent_attention_kernel<float>, dim3(p.heads, T), dim3(256), shm, st, p);
+    else
+        hipLaunchKernelGGL(latent_attention_kernel<uint16_t>, dim3(p.heads, T), dim3(256), shm, st, p);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// ------------------------------------------------------------------ per-head output gate
+// v[t, h, :] *= sigmoid(gate[t, h]); gate logits sit in the projection row at column g_col
+__global__ __launch_bounds__(256) void head_gate_kernel(float* v, const float* proj, int64_t ld, int g_col, int heads, int vd,
+                                                        int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int64_t t = i / ((int64_t)heads * vd);
+    const int h = (int)((i / vd) % heads);
+    const float g = proj[t * ld + g_col + h];
+    v[i] *= 1.0f / (1.0f + expf(-g));
+}
+int head_gate(float* v, const float* proj, int64_t ld, int g_col, int heads, int vd, int T, hipStream_t st) {
+    const int64_t n = (int64_t)T * heads * vd;
+    hipLaunchKernelGGL(head_gate_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, v, proj, ld, g_col, heads, vd, n);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// ------------------------------------------------------------------ norm on the sublayer output
+__global__ __launch_bounds__(256) void postnorm_add_kernel(const float* x, const float* v, float* y, int W, float gain,
+                                                           float eps) {
+    __shared__ float red[4];
+    const int64_t t = blockIdx.x;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < W; i += 256) {
+        const float a = v[t * W + i];
+        ss += a * a;
+    }
+    ss = block_sum256(ss, red);
+    const float inv = gain / sqrtf(ss / (float)W + eps);
+    for (int i = threadIdx.x; i < W; i += 256) y[t * W + i] = (x ? x[t * W + i] : 0.f) + v[t * W + i] * inv;
+}
+int postnorm_add(const float* x, const float* v, float* y, int T, int W, float gain, float eps, hipStream_t st) {
+    hipLaunchKernelGGL(postnorm_add_kernel, dim3(T), dim3(256), 0, st, x, v, y, W, gain, eps);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// rows picked by index, normed with one gain: out[i] = gain * x[rows[i]] / rms
+__global__ __launch_bounds__(256) void final_rows_kernel(const float* x, const int32_t* rows, float* out, int W, float gain,
+                                                         float eps) {
+    __shared__ float red[4];
+    const int64_t t = rows[blockIdx.x];
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < W; i += 256) {
+        const float a = x[t * W + i];
+        ss += a * a;
+    }
+    ss = block_sum256(ss, red);
+    const float inv = gain / sqrtf(ss / (float)W + eps);
+    for (int i = threadIdx.x; i < W; i += 256) out[(int64_t)blockIdx.x * W + i] = x[t * W + i] * inv;
+}
+int final_rows(const float* x, const int32_t* rows, float* out, int n, int W, float gain, float eps, hipStream_t st) {
+    hipLaunchKernelGGL(final_rows_kernel, dim3(n), dim3(256), 0, st, x, rows, out, W, gain, eps);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// ------------------------------------------------------------------ depth-weighted average
+// x[t, w] = sum_{j < n} a[j] X[j][t, w]; X[j] at stack + j * stride
+__global__ __launch_bounds__(256) void depth_mix_kernel(const float* stack, int64_t stride, const float* a, int n, float* x,
+                                                        int64_t count) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count) return;
+    float s = 0.f;
+    for (int j = 0; j < n; j++) s = fmaf(a[j], stack[j * stride + i], s);
+    x[i] = s;
+}
+int depth_mix(const float* stack, int64_t stride, const float* a, int n, float* x, int64_t count, hipStream_t st) {
+    hipLaunchKernelGGL(depth_mix_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st, stack, stride, a, n, x, count);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// ------------------------------------------------------------------ gated activation
+// a[m, j] = silu(gu[m, j]) * gu[m, ff + j]
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float* gu, float* a, int ff, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int64_t m = i / ff;
+    const int j = (int)(i % ff);
+    const float g = gu[m * 2 * ff + j], u = gu[m * 2 * ff + ff + j];
+    a[i] = g / (1.0f + expf(-g)) * u;
+}
+int silu_mul(const float* gu, float* a, int64_t M, int ff, hipStream_t st) {
+    const int64_t n = M * ff;
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, gu, a, ff, n);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// ------------------------------------------------------------------ mixture of experts
+// Router: z = W_r y in fp32, s = sigmoid(z); the `top` largest (ties: the lower index) in
+// descending order -> sel[t, k], score[t, k].  One block per row.
+template <typename TW>
+__global__ __launch_bounds__(256) void route_kernel(const float* y, const TW* Wr, int W, int E, int top, int32_t* sel,
+                                                    float* score) {
+    extern __shared__ float s[];   // [E]
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int e = wave; e < E; e += 4) {
+        float z = 0.f;
+        for (int i = lane; i < W; i += 64) z = fmaf(y[t * W + i], ldf<TW>(Wr, (int64_t)e * W + i), z);
+        z = wave_sum(z);
+        if (lane == 0) s[e] = 1.0f / (1.0f + expf(-z));
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int k = 0; k < top; k++) {
+            int best = 0;
+            float bv = -1.f;
+            for (int e = 0; e < E; e++)
+                if (s[e] > bv) {
+                    bv = s[e];
+                    best = e;
+                }
+            sel[t * top + k] = best;
+            score[t * top + k] = bv;
+            s[best] = -2.f;
+        }
+    }
+}
+int route_sigmoid_topk(const float* y, const void* Wr, bool w_f32, int T, int W, int E, int top, int32_t* sel, float* score,
+                       hipStream_t st) {
+    QIE_REQUIRE(top >= 1 && top <= E && E <= 8192, "router: top %d of %d experts", top, E);
+    if (w_f32)
+        hipLaunchKernelGGL(route_kernel<float>, dim3(T), dim3(256), (size_t)E * 4, st, y, (const float*)Wr, W, E, top, sel, score);
+    else
+        hipLaunchKernelGGL(route_kernel<uint16_t>, dim3(T), dim3(256), (size_t)E * 4, st, y, (const uint16_t*)Wr, W, E, top, sel,
+                           score);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// Grouping: entries i = t * top + k in index order, gathered per expert.  cnt[e] first, then
+// off[e] = sum of the counts before e and slot_of[i] = off[sel[i]] + rank of i among its expert's.
+__global__ __launch_bounds__(256) void moe_count_kernel(const int32_t* sel, int n, int32_t* cnt) {
+    __shared__ int red[4];
+    const int e = blockIdx.x;
+    int c = 0;
+    for (int i = threadIdx.x; i < n; i += 256) c += sel[i] == e;
+    for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, 64);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) cnt[e] = red[0] + red[1] + red[2] + red[3];
+}
+__global__ __launch_bounds__(256) void moe_fill_kernel(const int32_t* sel, int n, const int32_t* cnt, int E, int32_t* off,
+                                                       int32_t* slot_of) {
+    __shared__ int wsum[4];
+    __shared__ int base_s;
+    const int e = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    if (tid == 0) {
+        int o = 0;
+        for (int i = 0; i < e; i++) o += cnt[i];
+        base_s = o;
+        off[e] = o;
+        if (e == E - 1) off[E] = o + cnt[e];
+    }
+    __syncthreads();
+    int base = base_s;
+    for (int i0 = 0; i0 < n; i0 += 256) {
+        const int i = i0 + tid;
+        const bool f = i < n && sel[i] == e;
+        const unsigned long long b = __ballot(f);
+        const int before = __popcll(b & ((1ull << lane) - 1ull));
+        if (lane == 0) wsum[wave] = __popcll(b);
+        __syncthreads();
+        int wb = 0;
+        for (int w = 0; w < wave; w++) wb += wsum[w];
+        if (f) slot_of[i] = base + wb + before;
+        base += wsum[0] + wsum[1] + wsum[2] + wsum[3];
+        __syncthreads();
+    }
+}
+int moe_group(const int32_t* sel, int n, int E, int32_t* cnt, int32_t* off, int32_t* slot_of, hipStream_t st) {
+    hipLaunchKernelGGL(moe_count_kernel, dim3(E), dim3(256), 0, st, sel, n, cnt);
+    QIE_LAUNCH_CHECK();
+    hipLaunchKernelGGL(moe_fill_kernel, dim3(E), dim3(256), 0, st, sel, n, cnt, E, off, slot_of);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+// xg[slot_of[i], :] = score[i] * y[i / top, :]
+__global__ __launch_bounds__(256) void moe_gather_kernel(const float* y, const float* score, const int32_t* slot_of, int top, int W,
+                                                         float* xg) {
+    const int64_t i = blockIdx.x;
+    const int64_t t = i / top, d = slot_of[i];
+    const float s = score[i];
+    for (int w = threadIdx.x; w < W; w += 256) xg[d * W + w] = s * y[t * W + w];
+}
+int moe_gather(const float* y, const float* score, const int32_t* slot_of, int T, int top, int W, float* xg, hipStream_t st) {
+    hipLaunchKernelGGL(moe_gather_kernel, dim3(T * top), dim3(256), 0, st, y, score, slot_of, top, W, xg);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+// f[t, :] = sum_k yd[slot_of[t * top + k], :]
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* yd, const int32_t* slot_of, int top, int W, float* f) {
+    const int64_t t = blockIdx.x;
+    for (int w = threadIdx.x; w < W; w += 256) {
+        float s = 0.f;
+        for (int k = 0; k < top; k++) s += yd[(int64_t)slot_of[t * top + k] * W + w];
+        f[t * W + w] = s;
+    }
+}
+int moe_combine(const float* yd, const int32_t* slot_of, int T, int top, int W, float* f, hipStream_t st) {
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, st, yd, slot_of, top, W, f);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// ------------------------------------------------------------------ conversions
+__global__ __launch_bounds__(256) void rows_to_bf16_kernel(const float* x, uint16_t* y, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) y[i] = f2bf(x[i]);
+}
+int rows_to_bf16(const float* x, uint16_t* y, int64_t n, hipStream_t st) {
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(rows_to_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, x, y, n);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+__global__ __launch_bounds__(256) void bf16_to_f32_kernel(const uint16_t* x, float* y, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) y[i] = bf2f(x[i]);
+}
+int bf16_to_f32(const uint16_t* x, float* y, int64_t n, hipStream_t st) {
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(bf16_to_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, x, y, n);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // namespace lay
+}  // namespace qie

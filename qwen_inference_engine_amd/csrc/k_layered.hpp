@@ -1,0 +1,83 @@
+// k_layered.hpp — launchers of the layered-model kernels (k_layered.hip).  Host functions take
+// a stream, never allocate or synchronise, and return 0 or an error with qie_last_error() text.
+#pragma once
+
+#include "qie_common.hpp"
+
+namespace qie {
+namespace lay {
+
+// y[m, n] = sum_k A[m, k] W[n, k] (+ batch z: A + z sA, W + z sW, Y + z sY).  A fp32, rounded to
+// bf16 on load when round_a; W fp32 or bf16 words; Y fp32.  grp_off (device, batch + 1 entries):
+// batch z covers rows [grp_off[z], grp_off[z + 1]) of A and Y (M is then the largest row count a
+// group can have); the k loop of an element is the same whatever else the launch holds.
+struct LinearP {
+    const float* A;
+    int64_t lda;
+    const void* W;
+    int64_t ldw;
+    float* Y;
+    int64_t ldy;
+    int M, N, K, batch;
+    int64_t sA, sW, sY;
+    int round_a;
+    const int32_t* grp_off;
+};
+int linear(const LinearP& p, bool w_f32, hipStream_t st);
+
+// Paged latent cache: page p at pool + p * page_stride elements; inside a page the rows of one
+// caching layer start at layer_off and are D = R + rot wide: [c (R) | rotated shared key (rot)].
+// Token t of slot s is row t % page_tokens of page table[s * max_pages + t / page_tokens].
+struct LatentCache {
+    void* pool;
+    int64_t page_stride;
+    const int32_t* table;
+    int page_tokens, max_pages;
+};
+
+struct LatentPostP {
+    float* proj;          // [T][ld]: q heads, then (own_kv) the compressed row and the shared key part
+    int64_t ld;
+    const int32_t* row_slot;
+    const int32_t* row_pos;
+    int heads, dim, rot, rot_dims, R, own_kv;
+    const float* norm_w;  // [R]
+    float eps;
+    const float* rope_cos;   // [positions][rot_dims / 2]
+    const float* rope_sin;
+    LatentCache cache;
+    int64_t layer_off;
+};
+int latent_post(const LatentPostP& p, bool cache_f32, int T, hipStream_t st);
+
+struct LatentAttnP {
+    const float* q_abs;   // [T][heads][R]
+    const float* proj;    // rotated query parts are read from the projection rows
+    int64_t ld;
+    const int32_t* row_slot;
+    const int32_t* row_pos;
+    int heads, dim, rot, R, window;
+    float scale;
+    LatentCache cache;
+    int64_t layer_off;
+    float* out;           // [T][heads][R]
+};
+int latent_attention(const LatentAttnP& p, bool cache_f32, int T, hipStream_t st);
+
+int embed_rows(const void* E, bool w_f32, const int32_t* tok, float* out, int T, int W, int vocab, hipStream_t st);
+int head_gate(float* v, const float* proj, int64_t ld, int g_col, int heads, int vd, int T, hipStream_t st);
+// y = (x ? x : 0) + gain * v / sqrt(mean(v^2) + eps), rows of W
+int postnorm_add(const float* x, const float* v, float* y, int T, int W, float gain, float eps, hipStream_t st);
+int final_rows(const float* x, const int32_t* rows, float* out, int n, int W, float gain, float eps, hipStream_t st);
+int depth_mix(const float* stack, int64_t stride, const float* a, int n, float* x, int64_t count, hipStream_t st);
+int silu_mul(const float* gu, float* a, int64_t M, int ff, hipStream_t st);
+int route_sigmoid_topk(const float* y, const void* Wr, bool w_f32, int T, int W, int E, int top, int32_t* sel, float* score,
+                       hipStream_t st);
+int moe_group(const int32_t* sel, int n, int E, int32_t* cnt, int32_t* off, int32_t* slot_of, hipStream_t st);
+int moe_gather(const float* y, const float* score, const int32_t* slot_of, int T, int top, int W, float* xg, hipStream_t st);
+int moe_combine(const float* yd, const int32_t* slot_of, int T, int top, int W, float* f, hipStream_t st);
+int rows_to_bf16(const float* x, uint16_t* y, int64_t n, hipStream_t st);
+int bf16_to_f32(const uint16_t* x, float* y, int64_t n, hipStream_t st);
+
+}  // namespace lay
+}  // namespace qie

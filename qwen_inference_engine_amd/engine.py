@@ -16,7 +16,7 @@ from typing import Dict, List, Optional, Sequence
 import numpy as np
 
 from . import _lib
-from .spec import ModelSpec
+from .spec import LayeredSpec, ModelSpec
 from .weights import SynthParams
 
 REF_PREFILL_SAMPLING = dict(top_k=50, temperature=1.0, seed=1234)   # qwen_main.cu:241
@@ -141,9 +141,18 @@ class Comm:
 class Engine:
     def __init__(self, spec: ModelSpec, device: int = 0, max_ctx: int = 4096, use_graph: bool = True,
                  comm: Optional[Comm] = None, weight_fp8: bool = False, comm_always: bool = False,
-                 prefill_fp8: bool = False):
+                 prefill_fp8: bool = False, dtype: str = "bfloat16"):
+        """spec: a ModelSpec (the Qwen decoder) or a LayeredSpec (a model given layer by layer;
+        its tensors come through load_tensors / load_dir).  dtype "float32" (layered engines
+        only) computes everything in true fp32."""
         self.lib = _lib.load()
         self.spec = spec
+        self.layered = isinstance(spec, LayeredSpec)
+        if dtype not in ("bfloat16", "float32"):
+            raise ValueError(f"dtype {dtype!r}: bfloat16 or float32")
+        if dtype == "float32" and not self.layered:
+            raise ValueError("float32 compute is implemented for layered engines only")
+        self.dtype = dtype
         self._spec_c = spec.to_c()
         opts = _lib.EngineOptsC()
         opts.device, opts.max_ctx, opts.use_graph = device, max_ctx, int(use_graph)
@@ -154,14 +163,51 @@ class Engine:
         # numerics flag: prefill projections on the block-scaled fp8 MFMA (activations quantised
         # per row to e4m3; needs weight_fp8) — the oracle's Model(prefill_act_fp8=True)
         opts.prefill_fp8 = int(prefill_fp8)
+        opts.compute_f32 = int(dtype == "float32")
         self.comm = comm
         self._fp8 = weight_fp8
         h = C.c_void_p()
-        _lib.check(self.lib.qie_engine_create(C.byref(self._spec_c), C.byref(opts), C.byref(h)),
-                   "qie_engine_create")
+        if self.layered:
+            arch, self._arch_keep = self._spec_c
+            _lib.check(self.lib.qie_engine_create_layered(C.byref(arch), C.byref(opts), C.byref(h)),
+                       "qie_engine_create_layered")
+        else:
+            _lib.check(self.lib.qie_engine_create(C.byref(self._spec_c), C.byref(opts), C.byref(h)),
+                       "qie_engine_create")
         self.h = h
         self.max_ctx = max_ctx
         self._keep = None
+
+    # ------------------------------------------------------------ layered engines
+    def load_tensors(self, tensors) -> "Engine":
+        """Layered engines: {name: array or (dtype code, array)} -> device weights.  uint16
+        arrays are bf16 words, float32 / int32 arrays themselves.  Tensors the architecture does
+        not name are ignored; a missing one or a wrong shape raises."""
+        if not self.layered:
+            raise ValueError("load_tensors: layered engines only")
+        need = self.spec.tensor_shapes()
+        codes = {np.dtype(np.uint16): 0, np.dtype(np.int32): 1, np.dtype(np.float32): 2}
+        for name in need:
+            if name not in tensors:
+                raise KeyError(f"checkpoint has no tensor {name!r}")
+            t = tensors[name]
+            a = t[1] if isinstance(t, tuple) else t
+            a = np.asarray(a)
+            dims = a.shape                      # (ascontiguousarray turns a 0-d array into [1])
+            a = np.ascontiguousarray(a)
+            if a.dtype not in codes:
+                raise TypeError(f"tensor {name!r}: dtype {a.dtype} (bf16 words as uint16, float32 or int32)")
+            shape = (C.c_int64 * max(len(dims), 1))(*dims)
+            _lib.check(self.lib.qie_engine_put_tensor(self.h, name.encode(), a.ctypes.data, codes[a.dtype], len(dims), shape),
+                       f"qie_engine_put_tensor({name})")
+        _lib.check(self.lib.qie_engine_finalize_weights(self.h), "qie_engine_finalize_weights")
+        return self
+
+    def load_dir(self, path: str) -> "Engine":
+        """Layered engines: the model.safetensors of a model folder."""
+        import os
+        from .weights import read_safetensors
+        return self.load_tensors(read_safetensors(os.path.join(path, "model.safetensors")))
 
     def init_synthetic(self, p: SynthParams = SynthParams()) -> "Engine":
         _lib.check(self.lib.qie_engine_init_synthetic(self.h, p.seed, p.w_scale, p.norm_scale, p.bias_scale),
@@ -232,6 +278,8 @@ class Batch:
         self.lib = engine.lib
         self.B = batch
         self.max_ctx = max_ctx
+        if engine.layered and page_tokens is None:
+            page_tokens = 64                    # layered engines are always paged
         self.paged = page_tokens is not None
         h = C.c_void_p()
         if self.paged:
@@ -240,6 +288,51 @@ class Batch:
         else:
             _lib.check(self.lib.qie_batch_create(engine.h, batch, max_ctx, C.byref(h)), "qie_batch_create")
         self.h = h
+
+    # ------------------------------------------------------------ ragged steps (layered engines)
+    def step(self, entries: Sequence[tuple], want: Sequence[int] = (), fetch: bool = True) -> Optional[np.ndarray]:
+        """One step over [(slot, token ids), ...]: every entry continues its slot (a fresh or
+        released slot starts at position 0), portions of prompts beside single tokens.  want:
+        indices into the step's rows (entries laid end to end) whose logits are computed;
+        returns them as float32 [len(want), vocab] (None when fetch is False: they stay on the
+        device for step_sample)."""
+        slots = np.asarray([int(s) for s, _ in entries], dtype=np.int32)
+        counts = np.asarray([len(t) for _, t in entries], dtype=np.int32)
+        toks = np.ascontiguousarray(np.concatenate([np.asarray(t, dtype=np.int32).reshape(-1) for _, t in entries]))
+        w = np.ascontiguousarray(np.asarray(list(want), dtype=np.int32))
+        out = np.zeros((len(w), self.e.spec.vocab), dtype=np.float32) if fetch and len(w) else None
+        p32 = C.POINTER(C.c_int32)
+        _lib.check(self.lib.qie_batch_step(
+            self.h, len(slots), slots.ctypes.data_as(p32), counts.ctypes.data_as(p32), toks.ctypes.data_as(p32),
+            len(w), w.ctypes.data_as(p32) if len(w) else None,
+            out.ctypes.data_as(C.POINTER(C.c_float)) if out is not None else None), "qie_batch_step")
+        self._last_want = len(w)
+        return out
+
+    def step_sample(self, sampling: Sampling = GREEDY) -> List[int]:
+        """One sampled id per wanted row of the last step."""
+        n = getattr(self, "_last_want", 0)
+        out = (C.c_int32 * max(n, 1))()
+        sc = sampling.to_c()
+        _lib.check(self.lib.qie_batch_step_sample(self.h, C.byref(sc), out), "qie_batch_step_sample")
+        return list(out)[:n]
+
+    def keep_layers(self, on: bool = True) -> None:
+        _lib.check(self.lib.qie_batch_keep_layers(self.h, int(on)), "qie_batch_keep_layers")
+
+    def step_layers(self, rows: int) -> np.ndarray:
+        """The residual stream after every layer of the last step, float32 [layers, rows, width]
+        (after keep_layers())."""
+        out = np.zeros((self.e.spec.n_layers, rows, self.e.spec.width), dtype=np.float32)
+        _lib.check(self.lib.qie_batch_step_layers(self.h, out.ctypes.data_as(C.POINTER(C.c_float)), out.size),
+                   "qie_batch_step_layers")
+        return out
+
+    def time_stage(self, which: int, layer: int = 0, iters: int = 20) -> float:
+        """Microseconds per run of one stage at the last step's shape (qie_batch_time_stage)."""
+        us = C.c_double()
+        _lib.check(self.lib.qie_batch_time_stage(self.h, which, layer, iters, C.byref(us)), "qie_batch_time_stage")
+        return us.value
 
     def prefill(self, seq: int, ids: Sequence[int], sampling: Sampling = GREEDY) -> int:
         arr = (C.c_int32 * len(ids))(*[int(i) for i in ids])

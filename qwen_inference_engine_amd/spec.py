@@ -11,6 +11,9 @@ from __future__ import annotations
 import dataclasses
 import json
 
+from typing import List, Optional, Tuple
+
+from . import _lib
 from ._lib import ModelSpecC, QIE_NUMERICS_HF, QIE_NUMERICS_REF
 
 REF_EPS = 1e-4        # normalization.cu:9, qk_norm.cu:46
@@ -159,3 +162,167 @@ def tp_shardable(spec: ModelSpec, tp: int):
     if spec.vocab % tp:
         return False, f"vocab {spec.vocab} not divisible by {tp}"
     return True, ""
+
+
+# ------------------------------------------------------------------ layered models
+# Models given as a list of layers, each with its own mixer and feed-forward (the engine tier of
+# qie_engine_create_layered).  A config.json of such a model names its design in "architecture";
+# ARCHITECTURES maps that name to the reader of the config.
+
+@dataclasses.dataclass(frozen=True)
+class LatentAttention:
+    """Mixer: latent (compressed-KV) attention over a sliding window with a per-head output gate."""
+    heads: int
+    dim: int          # unrotated query / key coordinates per head
+    rot_dim: int      # rotated coordinates per head (the key's are shared by all heads)
+    vdim: int
+    kv_rank: int
+    window: int
+    rot_dims: int     # rotated coordinates that actually turn (rotate-half pairs i, i + rot_dims / 2)
+    rot_base: float
+    scale: float
+    kv_from: Optional[int] = None   # the layer whose cache rows this layer reads
+
+
+@dataclasses.dataclass(frozen=True)
+class FeedForward:
+    kind: str         # "dense" or "moe"
+    ff: int           # hidden size (of one expert for "moe")
+    experts: int = 0
+    top: int = 0
+
+
+@dataclasses.dataclass(frozen=True)
+class LayerSpec:
+    mixer: LatentAttention
+    mlp: Optional[FeedForward]
+
+
+@dataclasses.dataclass(frozen=True)
+class LayeredSpec:
+    name: str
+    width: int
+    vocab: int
+    norm_eps: float
+    layers: Tuple[LayerSpec, ...]
+    depth_mix: bool = True
+
+    @property
+    def n_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def hidden(self) -> int:
+        return self.width
+
+    def to_c(self):
+        """(ArchDescC, keepalive of its layer array)."""
+        arr = (_lib.LayerDescC * len(self.layers))()
+        for d, L in zip(arr, self.layers):
+            m = L.mixer
+            d.mixer = _lib.QIE_MIXER_LATENT_ATTENTION
+            d.heads, d.dim, d.rot_dim, d.vdim, d.kv_rank = m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank
+            d.window, d.kv_from, d.rot_dims = m.window, -1 if m.kv_from is None else m.kv_from, m.rot_dims
+            d.rot_base, d.scale = m.rot_base, m.scale
+            if L.mlp is None:
+                d.ff_kind = _lib.QIE_FF_NONE
+            elif L.mlp.kind == "dense":
+                d.ff_kind, d.ff = _lib.QIE_FF_DENSE, L.mlp.ff
+            else:
+                d.ff_kind, d.ff, d.experts, d.top = _lib.QIE_FF_MOE, L.mlp.ff, L.mlp.experts, L.mlp.top
+        a = _lib.ArchDescC()
+        a.n_layers, a.width, a.vocab, a.norm_eps = len(self.layers), self.width, self.vocab, self.norm_eps
+        a.depth_mix = int(self.depth_mix)
+        a.layers = arr
+        return a, arr
+
+    def tensor_shapes(self) -> "dict[str, List[int]]":
+        """Checkpoint tensor names and shapes of this architecture."""
+        W, out = self.width, {"embed": [self.vocab, self.width]}
+        for i, L in enumerate(self.layers):
+            m, p = L.mixer, f"l{i}."
+            out[p + "norm1"] = []
+            if L.mlp is not None:
+                out[p + "norm2"] = []
+            out[p + "mix.q"] = [m.heads * (m.dim + m.rot_dim), W]
+            if m.kv_from is None:
+                out[p + "mix.dkv"] = [m.kv_rank + m.rot_dim, W]
+                out[p + "mix.dkv.norm"] = [m.kv_rank]
+            out[p + "mix.uk"] = [m.heads * m.dim, m.kv_rank]
+            out[p + "mix.uv"] = [m.heads * m.vdim, m.kv_rank]
+            out[p + "mix.g"] = [m.heads, W]
+            out[p + "mix.o"] = [W, m.heads * m.vdim]
+            if L.mlp is not None and L.mlp.kind == "dense":
+                out.update({p + "mlp.gate": [L.mlp.ff, W], p + "mlp.up": [L.mlp.ff, W], p + "mlp.down": [W, L.mlp.ff]})
+            elif L.mlp is not None:
+                for e in range(L.mlp.experts):
+                    q = f"{p}mlp.e{e}."
+                    out.update({q + "gate": [L.mlp.ff, W], q + "up": [L.mlp.ff, W], q + "down": [W, L.mlp.ff]})
+                out[p + "mlp.router"] = [L.mlp.experts, W]
+            if self.depth_mix:
+                out[p + "dwa"] = [i + 2]
+        out["final.norm"] = []
+        out["head"] = [self.vocab, W]
+        return out
+
+    def cache_row_elems(self) -> int:
+        """Cached elements per token, all caching layers together."""
+        return sum(L.mixer.kv_rank + L.mixer.rot_dim for L in self.layers if L.mixer.kv_from is None)
+
+    def step_flops(self, rows: int, ctx: int) -> float:
+        """Multiply-adds x 2 of one step of `rows` tokens whose windows hold about `ctx` keys."""
+        W, f = self.width, 0.0
+        for L in self.layers:
+            m = L.mixer
+            n_in = m.heads * (m.dim + m.rot_dim) + m.heads + (m.kv_rank + m.rot_dim if m.kv_from is None else 0)
+            f += 2.0 * rows * W * n_in + 2.0 * rows * m.heads * m.kv_rank * (m.dim + m.vdim) + 2.0 * rows * W * m.heads * m.vdim
+            f += 2.0 * rows * m.heads * min(ctx, m.window) * (2 * m.kv_rank + m.rot_dim)
+            if L.mlp is not None:
+                k = 1 if L.mlp.kind == "dense" else L.mlp.top
+                f += 2.0 * rows * k * 3 * W * L.mlp.ff
+        return f + 2.0 * rows * W * self.vocab
+
+
+def _tivazen_from_config(cfg: dict, name: str) -> LayeredSpec:
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        if L["type"] != "latent_attention":
+            raise ValueError(f"layer {i}: unknown mixer type {L['type']!r}")
+        m = L["mixer"]
+        rot = m.get("rot") or {}
+        mixer = LatentAttention(
+            heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]), vdim=int(m["vdim"]),
+            kv_rank=int(m["kv_rank"]), window=int(m["mask"]["size"]), rot_dims=int(rot.get("dims", m["rot_dim"])),
+            rot_base=float(rot.get("base", 10000.0)), scale=float(m["scale"]),
+            kv_from=None if m.get("kv_from") is None else int(m["kv_from"]))
+        f = L.get("mlp")
+        if f is None:
+            mlp = None
+        elif f["kind"] == "dense":
+            mlp = FeedForward("dense", int(f["ff"]))
+        elif f["kind"] == "moe":
+            mlp = FeedForward("moe", int(f["expert"]["ff"]), int(f["router"]["experts"]), int(f["router"]["top"]))
+        else:
+            raise ValueError(f"layer {i}: unknown feed-forward kind {f['kind']!r}")
+        layers.append(LayerSpec(mixer, mlp))
+    return LayeredSpec(name, int(cfg["width"]), int(cfg["vocab"]), float(cfg["norm"]["eps"]), tuple(layers), True)
+
+
+ARCHITECTURES = {"Tivazen": _tivazen_from_config}
+
+
+def spec_from_config(cfg: dict, name: str = "model", numerics: str = "hf"):
+    """The spec class a config.json asks for: a layered design named by "architecture", else the
+    Qwen decoder (HuggingFace keys)."""
+    arch = cfg.get("architecture")
+    if arch is not None:
+        if arch not in ARCHITECTURES:
+            raise ValueError(f"unknown architecture {arch!r} (known: {sorted(ARCHITECTURES)})")
+        return ARCHITECTURES[arch](cfg, name)
+    return ModelSpec.from_hf_config(cfg, name=name, numerics=numerics)
+
+
+def spec_from_dir(path: str, numerics: str = "hf"):
+    import os
+    with open(os.path.join(path, "config.json")) as f:
+        return spec_from_config(json.load(f), name=os.path.basename(os.path.normpath(path)), numerics=numerics)

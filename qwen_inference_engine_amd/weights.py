@@ -123,6 +123,32 @@ def read_safetensors_header(path: str) -> Dict[str, dict]:
         return json.loads(f.read(n))
 
 
+_ST_DTYPES = {"BF16": (np.uint16, 0), "I32": (np.int32, 1), "F32": (np.float32, 2)}
+
+
+def read_safetensors(path: str) -> "Dict[str, Tuple[int, np.ndarray]]":
+    """Every tensor of one safetensors file as {name: (dtype code, array)}: code 0 = bf16 words
+    (uint16 array), 1 = int32, 2 = fp32 — the codes qie_engine_put_tensor takes.  The file is an
+    8-byte little-endian header length, that many bytes of JSON (name -> dtype, shape,
+    data_offsets relative to the end of the header) and the data."""
+    out = {}
+    with open(path, "rb") as f:
+        n = struct.unpack("<Q", f.read(8))[0]
+        hdr = json.loads(f.read(n))
+        base = 8 + n
+        for name, t in hdr.items():
+            if name == "__metadata__":
+                continue
+            if t["dtype"] not in _ST_DTYPES:
+                raise ValueError(f"{path}: tensor {name!r} has dtype {t['dtype']}, not one of {sorted(_ST_DTYPES)}")
+            np_t, code = _ST_DTYPES[t["dtype"]]
+            lo, hi = t["data_offsets"]
+            f.seek(base + lo)
+            a = np.frombuffer(f.read(hi - lo), dtype=np_t).reshape(t["shape"])
+            out[name] = (code, a)
+    return out
+
+
 def hf_tensor_shapes(spec: ModelSpec) -> "OrderedDict[str, List[int]]":
     H, hd, QD, KD, I, V = spec.hidden, spec.head_dim, spec.q_dim, spec.kv_dim, spec.ffn, spec.vocab
     d: "OrderedDict[str, List[int]]" = OrderedDict()
