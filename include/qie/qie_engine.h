@@ -307,8 +307,9 @@ int qie_engine_finalize_weights(qie_engine* e);
  * qie_batch_step_sample). */
 int qie_batch_step(qie_batch* b, int32_t n_entries, const int32_t* slots, const int32_t* counts, const int32_t* tokens,
                    int32_t n_want, const int32_t* want_rows, float* host_logits);
-/* Samples one id per wanted row of the last qie_batch_step (qie_sample on the rows, rounded to
- * bf16 as the sampler reads them); host_ids [n_want]. */
+/* Samples one id per wanted row of the last qie_batch_step; host_ids [n_want].  Greedy
+ * (top_k <= 1 or temperature <= 0): arg-max of the fp32 row, ties to the lowest id; otherwise
+ * qie_sample on the rows rounded to bf16, as the sampler reads them. */
 int qie_batch_step_sample(qie_batch* b, const qie_sampling* s, int32_t* host_ids);
 /* Diagnostics: enable != 0 makes every following step keep the stream after each layer;
  * qie_batch_step_layers copies the last step's [n_layers][rows][width] fp32 to host_out. */

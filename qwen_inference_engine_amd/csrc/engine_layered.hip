@@ -763,11 +763,16 @@ int qie_batch_step_sample(qie_batch* b, const qie_sampling* smp, int32_t* host_i
     qie_engine* e = b->e;
     hipStream_t st = e->stream;
     const int64_t V = e->lm->a.vocab;
-    QIE_TRY(lay::rows_to_bf16(s->logits, s->logits_bf, (int64_t)n * V, st));
-    std::vector<int32_t> steps(n, (int32_t)(s->steps & 0x7fffffff));
-    QIE_HIP(hipMemcpyAsync(s->d_step, steps.data(), (size_t)n * 4, hipMemcpyHostToDevice, st));
-    QIE_HIP(hipStreamSynchronize(st));
-    QIE_TRY(qie_sample(s->logits_bf, n, V, V, smp, s->d_step, s->d_ids, b->samp_ws, st));
+    if (smp->top_k <= 1 || !(smp->temperature > 0.f)) {
+        // greedy: on the fp32 rows themselves (two logits closer than a bf16 step stay apart)
+        QIE_TRY(lay::argmax_rows(s->logits, n, V, s->d_ids, st));
+    } else {
+        QIE_TRY(lay::rows_to_bf16(s->logits, s->logits_bf, (int64_t)n * V, st));
+        std::vector<int32_t> steps(n, (int32_t)(s->steps & 0x7fffffff));
+        QIE_HIP(hipMemcpyAsync(s->d_step, steps.data(), (size_t)n * 4, hipMemcpyHostToDevice, st));
+        QIE_HIP(hipStreamSynchronize(st));
+        QIE_TRY(qie_sample(s->logits_bf, n, V, V, smp, s->d_step, s->d_ids, b->samp_ws, st));
+    }
     QIE_HIP(hipMemcpyAsync(host_ids, s->d_ids, (size_t)n * 4, hipMemcpyDeviceToHost, st));
     QIE_HIP(hipStreamSynchronize(st));
     return 0;

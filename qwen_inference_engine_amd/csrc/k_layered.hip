@@ -497,6 +497,41 @@ int moe_combine(const float* yd, const int32_t* slot_of, int T, int top, int W, 
     return 0;
 }
 
+// ------------------------------------------------------------------ greedy choice on fp32 rows
+// ids[m] = the index of the largest logit of row m (ties: the lowest index).  One block per row.
+__global__ __launch_bounds__(256) void argmax_rows_kernel(const float* x, int64_t V, int32_t* ids) {
+    __shared__ float bv[256];
+    __shared__ int bi[256];
+    const float* r = x + (int64_t)blockIdx.x * V;
+    float v = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int64_t i = threadIdx.x; i < V; i += 256)
+        if (r[i] > v) {
+            v = r[i];
+            idx = (int)i;
+        }
+    bv[threadIdx.x] = v;
+    bi[threadIdx.x] = idx;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if ((int)threadIdx.x < o) {
+            const float w = bv[threadIdx.x + o];
+            const int j = bi[threadIdx.x + o];
+            if (w > bv[threadIdx.x] || (w == bv[threadIdx.x] && j < bi[threadIdx.x])) {
+                bv[threadIdx.x] = w;
+                bi[threadIdx.x] = j;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) ids[blockIdx.x] = bi[0] == 0x7fffffff ? 0 : bi[0];
+}
+int argmax_rows(const float* x, int M, int64_t V, int32_t* ids, hipStream_t st) {
+    hipLaunchKernelGGL(argmax_rows_kernel, dim3(M), dim3(256), 0, st, x, V, ids);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
 // ------------------------------------------------------------------ conversions
 __global__ __launch_bounds__(256) void rows_to_bf16_kernel(const float* x, uint16_t* y, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;

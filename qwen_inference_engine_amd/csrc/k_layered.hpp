@@ -76,6 +76,7 @@ int route_sigmoid_topk(const float* y, const void* Wr, bool w_f32, int T, int W,
 int moe_group(const int32_t* sel, int n, int E, int32_t* cnt, int32_t* off, int32_t* slot_of, hipStream_t st);
 int moe_gather(const float* y, const float* score, const int32_t* slot_of, int T, int top, int W, float* xg, hipStream_t st);
 int moe_combine(const float* yd, const int32_t* slot_of, int T, int top, int W, float* f, hipStream_t st);
+int argmax_rows(const float* x, int M, int64_t V, int32_t* ids, hipStream_t st);
 int rows_to_bf16(const float* x, uint16_t* y, int64_t n, hipStream_t st);
 int bf16_to_f32(const uint16_t* x, float* y, int64_t n, hipStream_t st);
 

@@ -11,6 +11,13 @@ prefill in one ``qie_prefill_batch`` pass), and retired at its stop token / toke
 slots run on the scratch page and their outputs are dropped), so the hipGraph captured
 for the batch is replayed unchanged.
 
+Layered engines (``Engine.layered``: models given layer by layer, stepped by ``Batch.step``)
+take the same admission, slots and page budget, but prompts are fed in portions: every step is
+ONE ragged engine step holding a single token for each decoding request and, within the
+``chunk_tokens`` budget of the step, the next portion of each prompt that is still being read
+(decoding requests first, then prompts in slot order).  A request's first token is sampled from
+the last row of its last portion.
+
 One sampling configuration per batcher (``qie_sampling`` is per step); slot rows are
 independent, so a request's tokens do not depend on what the other slots hold.
 """
@@ -34,6 +41,7 @@ class Request:
     slot: int = -1
     pages: int = 0
     done: bool = False
+    fed: int = 0            # prompt tokens already in the cache (ragged steps)
 
 
 def prefill_runs(admitted: Sequence[Request]) -> List[List[Request]]:
@@ -51,7 +59,11 @@ def prefill_runs(admitted: Sequence[Request]) -> List[List[Request]]:
 
 class ContinuousBatcher:
     def __init__(self, engine: Engine, slots: int = 8, max_ctx: Optional[int] = None, page_tokens: int = 128,
-                 n_pages: int = 0, sampling: Sampling = GREEDY, keep_logits: bool = False):
+                 n_pages: int = 0, sampling: Sampling = GREEDY, keep_logits: bool = False, chunk_tokens: int = 512):
+        self.ragged = bool(getattr(engine, "layered", False))
+        if chunk_tokens < 1:
+            raise ValueError("chunk_tokens must be positive")
+        self.chunk_tokens = chunk_tokens        # rows of one ragged step (layered engines)
         self.batch: Batch = engine.batch(slots, max_ctx, page_tokens=page_tokens, n_pages=n_pages)
         self.keep_logits = keep_logits          # copy each token's logit row (tests / diagnostics)
         self.max_ctx = self.batch.max_ctx
@@ -106,6 +118,8 @@ class ContinuousBatcher:
             self.budget -= need
             self.slots[free_slot] = r
             admitted.append(r)
+        if self.ragged:                         # prompts are read by the steps themselves
+            return
         # equal-length prompts landing in consecutive slots prefill in one pass
         # (qie_prefill_batch); tokens are emitted in admission order afterwards
         first: Dict[int, int] = {}
@@ -119,11 +133,56 @@ class ContinuousBatcher:
         for r in admitted:
             self._emit(r, first[r.rid], out, lg)
 
+    def plan(self) -> List[tuple]:
+        """The entries of the next ragged step, [(request, token ids, samples), ...]: one token
+        for every decoding request, then portions of unread prompts while the step's row budget
+        lasts; `samples` says whether the entry's last row yields the request's next token."""
+        entries, budget = [], self.chunk_tokens
+        live = [r for r in self.slots if r is not None]
+        for r in live:
+            if r.fed >= len(r.prompt):
+                entries.append((r, [r.tokens[-1]], True))
+                budget -= 1
+        for r in live:
+            if r.fed < len(r.prompt) and budget > 0:
+                n = min(budget, len(r.prompt) - r.fed)
+                entries.append((r, r.prompt[r.fed:r.fed + n], r.fed + n == len(r.prompt)))
+                budget -= n
+        entries.sort(key=lambda en: en[0].slot)
+        return entries
+
+    def _step_ragged(self, out: list) -> None:
+        entries = self.plan()
+        if not entries:
+            return
+        want, row = [], 0
+        for r, toks, samples in entries:
+            row += len(toks)
+            if samples:
+                want.append(row - 1)
+        lg = self.batch.step([(r.slot, toks) for r, toks, _ in entries], want, fetch=self.keep_logits)
+        ids = self.batch.step_sample(self.sampling) if want else []
+        k = 0
+        for r, toks, samples in entries:
+            if r.fed < len(r.prompt):
+                r.fed += len(toks)
+            if samples:
+                r.tokens.append(int(ids[k]))
+                if self.keep_logits:
+                    r.logits.append(lg[k].copy())
+                out.append((r.rid, int(ids[k])))
+                k += 1
+                if len(r.tokens) >= r.max_new_tokens or r.tokens[-1] in r.stop_ids:
+                    self._finish(r)
+
     def step(self) -> List[tuple]:
         """Admit what fits, then one decode step for every slot; returns the (request id,
         token) pairs produced, in slot order."""
         out: List[tuple] = []
         self._admit(out)
+        if self.ragged:
+            self._step_ragged(out)
+            return out
         if any(s is not None for s in self.slots):
             live = list(self.slots)
             ids = self.batch.decode_step(self.sampling)

@@ -1,0 +1,275 @@
+"""GPU: the layered engine tier (latent attention, routed experts, output-side scalar norms,
+depth-weighted residuals; ragged paged steps) against the plain numpy restatement in
+tests/layered_oracle.py, on small random models of several shapes.
+
+fp32 engines are held to REL32 of the logits' spread, bf16 engines to REL16 (bf16 operand
+rounding over a few layers).  Random weights are made peaky where a fault would otherwise hide:
+a larger attention scale or boosted queries make single keys carry visible weight.
+"""
+import numpy as np
+import pytest
+
+import layered_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+REL32 = 2e-4
+REL16 = 5e-2
+
+
+def words(a):
+    """float32 values that are exact bf16 -> bf16 words"""
+    return (np.ascontiguousarray(a, dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16).reshape(np.shape(a))
+
+
+def att(heads=3, dim=12, rot_dim=6, vdim=10, kv_rank=20, window=7, kv_from=None, mlp=None, base=100.0, scale=None):
+    d = dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=kv_rank, window=window, kv_from=kv_from, mlp=mlp,
+             base=base)
+    if scale is not None:
+        d["scale"] = scale
+    return d
+
+
+MIXED = [att(window=9, mlp=("dense", 28)),
+         att(window=5, kv_from=0, mlp=("moe", 14, 5, 2)),
+         att(heads=2, dim=8, rot_dim=8, vdim=16, kv_rank=24, window=33, mlp=None),
+         att(heads=2, dim=8, rot_dim=8, vdim=6, kv_rank=24, window=4, kv_from=2, mlp=("moe", 10, 3, 1))]
+
+
+class Model:
+    def __init__(self, layers, seed=0, vocab=101, width=40, dtype="float32", max_ctx=512, slots=4, page_tokens=16,
+                 n_pages=0, eps=1e-5, tweak=None):
+        import qwen_inference_engine_amd as q
+        self.rng = np.random.default_rng(seed)
+        self.cfg, self.T = O.random_model(self.rng, vocab=vocab, width=width, layers=layers, eps=eps)
+        if tweak is not None:
+            tweak(self.T)                       # values must stay exact bf16
+        self.spec = q.spec_from_config(self.cfg)
+        self.eng = q.Engine(self.spec, max_ctx=max_ctx, dtype=dtype).load_tensors({k: words(v) for k, v in self.T.items()})
+        self.batch = self.eng.batch(slots, max_ctx, page_tokens=page_tokens, n_pages=n_pages)
+        self.vocab, self.dtype = vocab, dtype
+        self.tol = REL32 if dtype == "float32" else REL16
+
+    def tokens(self, n):
+        return [int(t) for t in self.rng.integers(0, self.vocab, n)]
+
+    def ref(self, toks, layers_out=None):
+        return O.forward(self.cfg, self.T, toks, layers_out)
+
+    def close(self):
+        self.batch.close()
+        self.eng.close()
+
+
+def rel(got, want):
+    d = np.asarray(got, dtype=np.float64) - want
+    return float(np.abs(d).max() / (np.std(want) + 1e-30))
+
+
+def rel_most(got, want, q=0.9):
+    """The q-quantile over rows of the per-row root-mean-square error: a bf16 engine may pick another expert than
+    the oracle on a near-tie of router scores, which moves single rows by much more than rounding."""
+    d = np.sqrt(((np.asarray(got, dtype=np.float64) - want) ** 2).mean(axis=1))
+    return float(np.quantile(d, q) / (np.std(want) + 1e-30))
+
+
+def feed(m, slot, toks, cuts):
+    """Feeds toks to `slot` in portions of the sizes in `cuts` (then one by one); logits of all rows."""
+    out, pos = [], 0
+    sizes = list(cuts)
+    while pos < len(toks):
+        n = min(sizes.pop(0) if sizes else 1, len(toks) - pos)
+        out.append(m.batch.step([(slot, toks[pos:pos + n])], range(n)))
+        pos += n
+    return np.concatenate(out)
+
+
+@pytest.fixture
+def model():
+    made = []
+
+    def make(*a, **k):
+        made.append(Model(*a, **k))
+        return made[-1]
+    yield make
+    for m in made:
+        m.close()
+
+
+# ------------------------------------------------------------------ mechanisms, one at a time
+@pytest.mark.parametrize("layers", [
+    [att(mlp=None)],                                        # attention, output norm, depth mix alone
+    [att(rot_dim=0, mlp=None)],                             # no rotated part at all
+    [att(mlp=("dense", 28))],
+    [att(mlp=("moe", 14, 5, 2))],
+    [att(mlp=("moe", 14, 4, 4))],                           # every expert chosen
+    [att(mlp=None), att(kv_from=0, window=3, vdim=4, mlp=None)],   # borrowed cache rows, own window
+], ids=["attention", "no-rotary", "dense", "moe-top2", "moe-all", "kv-from"])
+def test_mechanism_streams_match_oracle(model, layers):
+    m = model(layers, seed=len(layers) + layers[0]["rot_dim"])
+    toks = m.tokens(23)
+    m.batch.keep_layers(True)
+    got = m.batch.step([(0, toks)], range(len(toks)))
+    want_layers = []
+    want = m.ref(toks, want_layers)
+    streams = m.batch.step_layers(len(toks))
+    for i, w in enumerate(want_layers):
+        assert rel(streams[i], w) < REL32, f"stream after layer {i}"
+    assert rel(got, want) < REL32
+
+
+def test_router_prefers_lower_index_on_equal_scores(model):
+    """Two identical router rows give equal scores: the lower expert index is chosen."""
+    def same_rows(T):
+        T["l0.mlp.router"][2] = T["l0.mlp.router"][0]
+        T["l0.mlp.router"][3] = T["l0.mlp.router"][1]
+    m = model([att(mlp=("moe", 14, 4, 1))], seed=5, tweak=same_rows)
+    toks = m.tokens(12)
+    assert rel(m.batch.step([(0, toks)], range(12)), m.ref(toks)) < REL32
+
+
+# ------------------------------------------------------------------ prompts, portions, decoding
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_whole_prompt_portions_and_decoding_agree(model, dtype):
+    m = model(MIXED, seed=11, dtype=dtype)
+    toks = m.tokens(90)
+    want = m.ref(toks)
+    err = rel if dtype == "float32" else rel_most
+    whole = m.batch.step([(0, toks)], range(len(toks)))
+    assert err(whole, want) < m.tol
+    # token by token from the first token on
+    single = feed(m, 1, toks, [])
+    assert err(single, want) < m.tol
+    # portions of changing size, down to two tokens, cut inside pages and windows
+    parts = feed(m, 2, toks, [2, 3, 11, 2, 17, 16, 2, 30])
+    assert err(parts, want) < m.tol
+    # the same position must not depend on the cut beyond rounding
+    bound = 1e-5 if dtype == "float32" else 2e-2
+    assert err(single, whole) < bound and err(parts, whole) < bound
+
+
+def test_unequal_requests_in_one_step_equal_each_alone(model):
+    m = model(MIXED, seed=12, slots=4)
+    reqs = [m.tokens(n) for n in (41, 7, 64, 18)]
+    want = [m.ref(t) for t in reqs]
+    # step 1: portions of different sizes; later steps: one decoding beside prompt portions
+    pos = [0, 0, 0, 0]
+    plan = [[(0, 16), (1, 7), (2, 33), (3, 2)], [(0, 1), (2, 31), (3, 16)], [(0, 24)]]
+    for step in plan:
+        entries, rows = [], []
+        for r, n in step:
+            entries.append((r, reqs[r][pos[r]:pos[r] + n]))
+        got = m.batch.step(entries, range(sum(n for _, n in step)))
+        row = 0
+        for r, n in step:
+            assert rel(got[row:row + n], want[r][pos[r]:pos[r] + n]) < REL32, (r, pos[r], n)
+            row += n
+            pos[r] += n
+
+
+def test_slots_and_pages_are_reused(model):
+    """A pool smaller than the sum of all requests: finished requests give their pages back
+    and later ones take the same slots and pages; stale rows must not leak."""
+    m = model(MIXED, seed=13, slots=2, page_tokens=16, n_pages=8)   # 7 pages = 112 tokens
+    free0, _, pt = m.batch.page_stats()
+    assert (free0, pt) == (7, 16)
+    for round_ in range(4):
+        a, b = m.tokens(60 + round_), m.tokens(37)
+        ga = m.batch.step([(0, a[:50]), (1, b)], range(50 + 37))
+        gb = m.batch.step([(0, a[50:])], range(len(a) - 50))
+        assert rel(np.concatenate([ga[:50], gb]), m.ref(a)) < REL32
+        assert rel(ga[50:], m.ref(b)) < REL32
+        with pytest.raises(Exception):
+            m.batch.step([(1, m.tokens(40))])         # 4 + 3 pages held: no room for 2 more
+        m.batch.release(0)
+        m.batch.release(1)
+        assert m.batch.page_stats()[0] == 7
+
+
+# ------------------------------------------------------------------ window edges, far keys
+def test_window_edges_in_prompt_and_decoding(model):
+    """Peaky attention (scale x 6): the key at distance window - 1 is seen, the one at distance
+    window is not — for windows shorter than, equal to and longer than a page."""
+    for window in (3, 16, 21):
+        layers = [att(window=window, scale=1.5, mlp=None), att(window=window + 2, scale=1.5, kv_from=0, mlp=None)]
+        m = model(layers, seed=20 + window, page_tokens=16)
+        toks = m.tokens(3 * window + 19)
+        want = m.ref(toks)
+        # the oracle itself must react to the edge (else this test shows nothing)
+        cfg2 = {**m.cfg, "layers": [{**L, "mixer": {**L["mixer"], "mask": {"size": L["mixer"]["mask"]["size"] + 1}}}
+                                    for L in m.cfg["layers"]]}
+        assert rel(O.forward(cfg2, m.T, toks), want) > 50 * REL32
+        assert rel(m.batch.step([(0, toks)], range(len(toks))), want) < REL32
+        cut = window + 5
+        assert rel(feed(m, 1, toks, [cut]), want) < REL32          # the window passes over decoded tokens
+
+
+def test_far_key_dominates_across_pages(model):
+    """Queries boosted 4x make single far keys dominate the softmax: the logits follow the
+    oracle while such a key is inside the window (several pages back) and after it has left."""
+    def boost(T):
+        T["l0.mix.q"] *= 4.0                    # a power of two keeps the values exact bf16
+    layers = [att(heads=2, dim=8, rot_dim=0, vdim=8, kv_rank=16, window=70, scale=1.0, mlp=None)]
+    m = model(layers, seed=31, width=24, page_tokens=16, max_ctx=256, tweak=boost)
+    toks = m.tokens(150)
+    want = m.ref(toks)
+    assert rel(m.batch.step([(0, toks)], range(150)), want) < REL32
+    assert rel(feed(m, 1, toks, [60]), want) < REL32           # 90 decoded tokens, the window leaves the prompt
+
+
+def test_first_tokens_and_single_token_request(model):
+    m = model(MIXED, seed=41)
+    for n in (1, 2, 3):
+        toks = m.tokens(n)
+        assert rel(m.batch.step([(0, toks)], range(n)), m.ref(toks)) < REL32
+        m.batch.release(0)
+
+
+def test_long_decoding_over_many_pages(model):
+    m = model([att(window=19, mlp=("moe", 14, 6, 2)), att(window=40, kv_from=0, mlp=("dense", 20))], seed=51,
+              page_tokens=16, max_ctx=400)
+    toks = m.tokens(330)
+    want = m.ref(toks)
+    assert rel(feed(m, 0, toks, [9]), want) < REL32
+
+
+def test_other_sizes_wide_latent_and_many_heads(model):
+    layers = [att(heads=5, dim=16, rot_dim=4, vdim=7, kv_rank=300, window=12, mlp=("moe", 9, 7, 3), base=50.0),
+              att(heads=1, dim=4, rot_dim=2, vdim=3, kv_rank=5, window=64, mlp=("dense", 130))]
+    m = model(layers, seed=61, vocab=67, width=52)
+    toks = m.tokens(70)
+    assert rel(feed(m, 0, toks, [33, 2, 20]), m.ref(toks)) < REL32
+
+
+# ------------------------------------------------------------------ generation through the scheduler
+def oracle_greedy(m, prompt, n):
+    toks, out = list(prompt), []
+    for _ in range(n):
+        t = int(np.argmax(m.ref(toks)[-1]))
+        out.append(t)
+        toks.append(t)
+    return out
+
+
+def test_greedy_generation_through_the_batcher(model):
+    """Five requests through ContinuousBatcher (two slots, a small page pool, 24-row steps):
+    prompts are read in portions beside decoding requests, finished requests free their slot
+    and pages for the waiting ones; greedy tokens equal the oracle's."""
+    from qwen_inference_engine_amd.scheduler import ContinuousBatcher
+    m = model(MIXED, seed=71, dtype="float32")
+    m.batch.close()
+    cb = ContinuousBatcher(m.eng, slots=2, max_ctx=128, page_tokens=16, n_pages=9, chunk_tokens=24, keep_logits=True)
+    m.batch = cb.batch                          # closed with the model, before its engine
+    prompts = [m.tokens(n) for n in (30, 5, 50, 1, 17)]
+    gens = [6, 9, 4, 7, 5]
+    rids = [cb.submit(p, g) for p, g in zip(prompts, gens)]
+    out = cb.run()
+    for p, g, rid in zip(prompts, gens, rids):
+        want = oracle_greedy(m, p, g)
+        got = out[rid]
+        assert len(got) == g
+        if got != want:   # a near-tie may flip: the kept logits must then be within rounding of the oracle's
+            k = next(i for i in range(g) if got[i] != want[i])
+            lg = m.ref(list(p) + want[:k])[-1]
+            assert abs(lg[got[k]] - lg[want[k]]) < 1e-4 * np.std(lg), (rid, k)
+    assert cb.batch.page_stats()[0] == 8
