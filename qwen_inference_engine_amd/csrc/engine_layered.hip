@@ -79,6 +79,9 @@ struct LayeredBatch {
           *y = nullptr, *gu = nullptr, *act = nullptr, *ffo = nullptr, *xg = nullptr, *yd = nullptr, *score = nullptr,
           *xn = nullptr, *logits = nullptr, *keep = nullptr;
     uint16_t* logits_bf = nullptr;
+    uint16_t* abf = nullptr;      // bf16 image of a product's left operand (bf16 engines: the MFMA / GEMV kernels read bf16)
+    int64_t m_abf = 0;            // its elements per row
+    std::vector<int32_t> h_off;   // host copy of the expert row offsets (prompt-sized steps)
     int32_t *row_slot = nullptr, *row_pos = nullptr, *tok = nullptr, *want = nullptr, *sel = nullptr, *cnt = nullptr,
             *off = nullptr, *slot_of = nullptr, *d_ids = nullptr, *d_step = nullptr;
     int32_t* h_stage = nullptr;   // pinned: row_slot, row_pos, tok of a step
@@ -286,6 +289,36 @@ static int lin(const qie_engine* e, const float* A, int64_t lda, const void* Wt,
     return lay::linear(p, e->lm->f32, e->stream);
 }
 
+// Row count from which a step's expert products run per expert on the MFMA kernels (one
+// device-to-host copy of the expert offsets per routed layer); below it the grouped kernel runs
+// without a host round trip.
+constexpr int kMoeSyncRows = 256;
+
+static bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+// y[M, N] = A[M, K] W[N, K]^T on the engine's bf16 kernels (MFMA GEMM, GEMV for few rows) when
+// the model runs bf16 operands and the shapes fit them (K a multiple of 8, 16-byte aligned
+// operands); `abf` receives the bf16 image of A, row stride K.  Else the plain kernel.
+static int dense_on(qie_batch* b, uint16_t* abf, bool staged, const float* A, int64_t lda, const void* Wt, float* Y, int64_t ldy,
+                    int M, int N, int K) {
+    const qie_engine* e = b->e;
+    if (!e->lm->f32 && abf && K % 8 == 0 && al16(Wt) && al16(abf)) {
+        if (!staged) QIE_TRY(lay::rows_to_bf16_strided(A, lda, abf, K, M, K, e->stream));
+        qie_linear_args a{};
+        a.x = abf; a.ldx = K;
+        a.w[0] = Wt; a.seg_rows[0] = N;
+        a.M = M; a.K = K; a.N = N;
+        a.y = Y; a.ldy = ldy;
+        a.epilogue = QIE_EPI_F32;
+        const int rc = qie_linear(&a, e->stream);
+        if (rc != -22) return rc;   // a shape those kernels do not take: the plain kernel below
+    }
+    return lin(e, A, lda, Wt, K, Y, ldy, M, N, K);
+}
+static int dense(qie_batch* b, const float* A, int64_t lda, const void* Wt, float* Y, int64_t ldy, int M, int N, int K) {
+    return dense_on(b, b->lb->abf, false, A, lda, Wt, Y, ldy, M, N, K);
+}
+
 static lay::LatentCache cache_of(const qie_batch* b) {
     return lay::LatentCache{b->kc, b->seq_stride, b->d_table, b->page_tokens, b->max_pages};
 }
@@ -295,7 +328,7 @@ static int enq_input_proj(qie_batch* b, int i, const float* xin, int T) {
     const LayeredModel* m = e->lm;
     const LayerDev& L = m->L[i];
     LayeredBatch* s = b->lb;
-    return lin(e, xin, m->a.width, L.w_in, m->a.width, s->proj, L.n_in, T, L.n_in, m->a.width);
+    return dense(b, xin, m->a.width, L.w_in, s->proj, L.n_in, T, L.n_in, m->a.width);
 }
 
 static int enq_latent_post(qie_batch* b, int i, int T) {
@@ -326,8 +359,23 @@ static int enq_absorb(qie_batch* b, int i, int T) {
     const qie_layer_desc& d = L.d;
     LayeredBatch* s = b->lb;
     const int hq = d.dim + d.rot_dim;
-    return lin(e, s->proj, L.n_in, L.uk_t, d.dim, s->qabs, (int64_t)d.heads * d.kv_rank, T, d.kv_rank, d.dim, d.heads, hq,
-               (int64_t)d.kv_rank * d.dim, d.kv_rank);
+    const int64_t HR = (int64_t)d.heads * d.kv_rank, HQ = (int64_t)d.heads * hq;
+    if (!e->lm->f32 && T > 16 && d.dim % 8 == 0 && hq % 8 == 0 && d.kv_rank % 4 == 0) {
+        // prompt-sized steps: one MFMA product per head on the bf16 image of the query rows
+        QIE_TRY(lay::rows_to_bf16_strided(s->proj, L.n_in, s->abf, HQ, T, (int)HQ, e->stream));
+        for (int h = 0; h < d.heads; h++) {
+            qie_linear_args a{};
+            a.x = s->abf + (int64_t)h * hq; a.ldx = HQ;
+            a.w[0] = (const uint16_t*)L.uk_t + (int64_t)h * d.kv_rank * d.dim; a.seg_rows[0] = d.kv_rank;
+            a.M = T; a.K = d.dim; a.N = d.kv_rank;
+            a.y = s->qabs + (int64_t)h * d.kv_rank; a.ldy = HR;
+            a.epilogue = QIE_EPI_F32;
+            QIE_TRY(qie_linear(&a, e->stream));
+        }
+        return 0;
+    }
+    return lin(e, s->proj, L.n_in, L.uk_t, d.dim, s->qabs, HR, T, d.kv_rank, d.dim, d.heads, hq, (int64_t)d.kv_rank * d.dim,
+               d.kv_rank);
 }
 
 static int enq_attention(qie_batch* b, int i, int T) {
@@ -357,10 +405,24 @@ static int enq_mixer_out(qie_batch* b, int i, int T) {
     const qie_layer_desc& d = L.d;
     LayeredBatch* s = b->lb;
     const int64_t HV = (int64_t)d.heads * d.vdim;
-    QIE_TRY(lin(e, s->olat, (int64_t)d.heads * d.kv_rank, L.uv, d.kv_rank, s->ov, HV, T, d.vdim, d.kv_rank, d.heads, d.kv_rank,
-                (int64_t)d.vdim * d.kv_rank, d.vdim));
+    const int64_t HR = (int64_t)d.heads * d.kv_rank;
+    if (!m->f32 && T > 16 && d.kv_rank % 8 == 0 && d.vdim % 4 == 0) {
+        QIE_TRY(lay::rows_to_bf16_strided(s->olat, HR, s->abf, HR, T, (int)HR, e->stream));
+        for (int h = 0; h < d.heads; h++) {
+            qie_linear_args a{};
+            a.x = s->abf + (int64_t)h * d.kv_rank; a.ldx = HR;
+            a.w[0] = (const uint16_t*)L.uv + (int64_t)h * d.vdim * d.kv_rank; a.seg_rows[0] = d.vdim;
+            a.M = T; a.K = d.kv_rank; a.N = d.vdim;
+            a.y = s->ov + (int64_t)h * d.vdim; a.ldy = HV;
+            a.epilogue = QIE_EPI_F32;
+            QIE_TRY(qie_linear(&a, e->stream));
+        }
+    } else {
+        QIE_TRY(lin(e, s->olat, HR, L.uv, d.kv_rank, s->ov, HV, T, d.vdim, d.kv_rank, d.heads, d.kv_rank,
+                    (int64_t)d.vdim * d.kv_rank, d.vdim));
+    }
     QIE_TRY(lay::head_gate(s->ov, s->proj, L.n_in, L.g_col, d.heads, d.vdim, T, e->stream));
-    return lin(e, s->ov, HV, L.wo, HV, s->mix, m->a.width, T, m->a.width, (int)HV);
+    return dense(b, s->ov, HV, L.wo, s->mix, m->a.width, T, m->a.width, (int)HV);
 }
 
 // feed-forward of layer i on rows y -> ffo
@@ -373,14 +435,38 @@ static int enq_ff(qie_batch* b, int i, int T) {
     const int W = m->a.width, ff = d.ff;
     hipStream_t st = e->stream;
     if (d.ff_kind == QIE_FF_DENSE) {
-        QIE_TRY(lin(e, s->y, W, L.w_gu, W, s->gu, 2 * ff, T, 2 * ff, W));
+        QIE_TRY(dense(b, s->y, W, L.w_gu, s->gu, 2 * ff, T, 2 * ff, W));
         QIE_TRY(lay::silu_mul(s->gu, s->act, T, ff, st));
-        return lin(e, s->act, ff, L.w_down, ff, s->ffo, W, T, W, ff);
+        return dense(b, s->act, ff, L.w_down, s->ffo, W, T, W, ff);
     }
     const int E = d.experts, top = d.top, n = T * top;
     QIE_TRY(lay::route_sigmoid_topk(s->y, L.w_router, m->f32, T, W, E, top, s->sel, s->score, st));
     QIE_TRY(lay::moe_group(s->sel, n, E, s->cnt, s->off, s->slot_of, st));
     QIE_TRY(lay::moe_gather(s->y, s->score, s->slot_of, T, top, W, s->xg, st));
+    if (!m->f32 && n >= kMoeSyncRows && W % 8 == 0 && ff % 8 == 0) {
+        // prompt-sized steps: the expert row ranges come to the host and every expert's rows go
+        // through the MFMA kernels; the products are the grouped kernel's, in another order
+        s->h_off.resize(E + 1);
+        QIE_HIP(hipMemcpyAsync(s->h_off.data(), s->off, (size_t)(E + 1) * 4, hipMemcpyDeviceToHost, st));
+        QIE_HIP(hipStreamSynchronize(st));
+        QIE_TRY(lay::rows_to_bf16_strided(s->xg, W, s->abf, W, n, W, st));
+        for (int x = 0; x < E; x++) {
+            const int r0 = s->h_off[x], cnt = s->h_off[x + 1] - r0;
+            if (cnt > 0)
+                QIE_TRY(dense_on(b, s->abf + (int64_t)r0 * W, true, s->xg + (int64_t)r0 * W, W,
+                                 (const uint16_t*)L.w_gu + (int64_t)x * 2 * ff * W, s->gu + (int64_t)r0 * 2 * ff, 2 * ff, cnt,
+                                 2 * ff, W));
+        }
+        QIE_TRY(lay::silu_mul(s->gu, s->act, n, ff, st));
+        QIE_TRY(lay::rows_to_bf16_strided(s->act, ff, s->abf, ff, n, ff, st));
+        for (int x = 0; x < E; x++) {
+            const int r0 = s->h_off[x], cnt = s->h_off[x + 1] - r0;
+            if (cnt > 0)
+                QIE_TRY(dense_on(b, s->abf + (int64_t)r0 * ff, true, s->act + (int64_t)r0 * ff, ff,
+                                 (const uint16_t*)L.w_down + (int64_t)x * W * ff, s->yd + (int64_t)r0 * W, W, cnt, W, ff));
+        }
+        return lay::moe_combine(s->yd, s->slot_of, T, top, W, s->ffo, st);
+    }
     QIE_TRY(lin(e, s->xg, W, L.w_gu, W, s->gu, 2 * ff, n, 2 * ff, W, E, 0, (int64_t)2 * ff * W, 0, s->off));
     QIE_TRY(lay::silu_mul(s->gu, s->act, n, ff, st));
     QIE_TRY(lin(e, s->act, ff, L.w_down, ff, s->yd, W, n, W, ff, E, 0, (int64_t)W * ff, 0, s->off));
@@ -428,18 +514,19 @@ static int enq_forward(qie_batch* b, int T, int n_want) {
     for (int i = 0; i < m->a.n_layers; i++) QIE_TRY(enq_layer(b, i, x, T, &x));
     if (n_want > 0) {
         QIE_TRY(lay::final_rows(x, s->want, s->xn, n_want, W, m->g_final, m->a.norm_eps, e->stream));
-        QIE_TRY(lin(e, s->xn, W, m->head, W, s->logits, m->a.vocab, n_want, m->a.vocab, W));
+        QIE_TRY(dense(b, s->xn, W, m->head, s->logits, m->a.vocab, n_want, m->a.vocab, W));
     }
     return 0;
 }
 
 static void lb_free(LayeredBatch* s) {
     void* ps[] = {s->stack, s->x, s->proj, s->qabs, s->olat, s->ov, s->mix, s->y, s->gu, s->act, s->ffo, s->xg, s->yd, s->score,
-                  s->row_slot, s->row_pos, s->tok, s->sel, s->cnt, s->off, s->slot_of, s->keep};
+                  s->row_slot, s->row_pos, s->tok, s->sel, s->cnt, s->off, s->slot_of, s->keep, s->abf};
     for (void* p : ps)
         if (p) hipFree(p);
     s->stack = s->x = s->proj = s->qabs = s->olat = s->ov = s->mix = s->y = s->gu = s->act = s->ffo = s->xg = s->yd = s->score =
         s->keep = nullptr;
+    s->abf = nullptr;
     s->row_slot = s->row_pos = s->tok = s->sel = s->cnt = s->off = s->slot_of = nullptr;
     s->cap = 0;
 }
@@ -476,6 +563,7 @@ static int ensure_rows(qie_batch* b, int64_t T) {
         A((void**)&s->row_slot, cap);
         A((void**)&s->row_pos, cap);
         A((void**)&s->tok, cap);
+        if (!m->f32) A((void**)&s->abf, cap * s->m_abf + 64, 2);
         if (s->keep_on) A((void**)&s->keep, L * cap * W);
         if (rc) return rc;
         s->cap = cap;
@@ -550,6 +638,8 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
             s->m_gu = std::max<int64_t>(s->m_gu, k * 2 * d.ff);
             s->m_act = std::max<int64_t>(s->m_act, k * d.ff);
         }
+        s->m_abf = std::max<int64_t>({s->m_abf, (int64_t)m->a.width, H * (d.dim + d.rot_dim), H * d.kv_rank, H * d.vdim,
+                                      d.ff_kind == QIE_FF_NONE ? 0 : k * std::max<int64_t>(d.ff, m->a.width)});
         if (d.ff_kind == QIE_FF_MOE) {
             s->m_top = std::max<int64_t>(s->m_top, d.top);
             s->m_e = std::max<int64_t>(s->m_e, d.experts);

@@ -543,6 +543,22 @@ int rows_to_bf16(const float* x, uint16_t* y, int64_t n, hipStream_t st) {
     QIE_LAUNCH_CHECK();
     return 0;
 }
+// y[m, k] = bf16(x[m, k]) for M rows of K values with row strides ldx / ldy
+__global__ __launch_bounds__(256) void rows_to_bf16_strided_kernel(const float* x, int64_t ldx, uint16_t* y, int64_t ldy, int K,
+                                                                   int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int64_t m = i / K;
+    const int k = (int)(i % K);
+    y[m * ldy + k] = f2bf(x[m * ldx + k]);
+}
+int rows_to_bf16_strided(const float* x, int64_t ldx, uint16_t* y, int64_t ldy, int64_t M, int K, hipStream_t st) {
+    const int64_t n = M * K;
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(rows_to_bf16_strided_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, x, ldx, y, ldy, K, n);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
 __global__ __launch_bounds__(256) void bf16_to_f32_kernel(const uint16_t* x, float* y, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n) y[i] = bf2f(x[i]);

@@ -78,6 +78,7 @@ int moe_gather(const float* y, const float* score, const int32_t* slot_of, int T
 int moe_combine(const float* yd, const int32_t* slot_of, int T, int top, int W, float* f, hipStream_t st);
 int argmax_rows(const float* x, int M, int64_t V, int32_t* ids, hipStream_t st);
 int rows_to_bf16(const float* x, uint16_t* y, int64_t n, hipStream_t st);
+int rows_to_bf16_strided(const float* x, int64_t ldx, uint16_t* y, int64_t ldy, int64_t M, int K, hipStream_t st);
 int bf16_to_f32(const uint16_t* x, float* y, int64_t n, hipStream_t st);
 
 }  // namespace lay
