@@ -81,6 +81,14 @@ struct LayeredBatch {
     uint16_t* logits_bf = nullptr;
     uint16_t* abf = nullptr;      // bf16 image of a product's left operand (bf16 engines: the MFMA / GEMV kernels read bf16)
     int64_t m_abf = 0;            // its elements per row
+    // matrix-core attention: row groups per head count, key-split partials
+    std::map<int, std::pair<int, int64_t>> groups;   // heads -> (group count, offset into d_groups) of this step
+    int4* d_groups = nullptr;
+    int64_t groups_cap = 0;
+    std::vector<int4> h_groups;
+    float *part_o = nullptr, *part_ml = nullptr;
+    int64_t part_cap = 0;         // (group, split) units the partials hold
+    bool interleaved = false;     // the cache pages carry the key-interleaved copy of c
     std::vector<int32_t> h_off;   // host copy of the expert row offsets (prompt-sized steps)
     int32_t *row_slot = nullptr, *row_pos = nullptr, *tok = nullptr, *want = nullptr, *sel = nullptr, *cnt = nullptr,
             *off = nullptr, *slot_of = nullptr, *d_ids = nullptr, *d_step = nullptr;
@@ -90,7 +98,7 @@ struct LayeredBatch {
     int64_t steps = 0;
     bool keep_on = false;
     // per-row maxima over the layers (scratch sizing)
-    int64_t m_in = 0, m_hr = 0, m_hv = 0, m_gu = 0, m_act = 0, m_top = 0, m_e = 0;
+    int64_t m_in = 0, m_hr = 0, m_hv = 0, m_gu = 0, m_act = 0, m_top = 0, m_e = 0, m_r = 0;
 };
 
 static inline float bf16_to_float(uint16_t h) {
@@ -350,6 +358,7 @@ static int enq_latent_post(qie_batch* b, int i, int T) {
     p.rope_sin = m->ropes[L.rope].sn;
     p.cache = cache_of(b);
     p.layer_off = s->layer_off[L.cache_layer];
+    p.interleaved = s->interleaved;
     return lay::latent_post(p, m->f32, T, e->stream);
 }
 
@@ -395,7 +404,77 @@ static int enq_attention(qie_batch* b, int i, int T) {
     p.cache = cache_of(b);
     p.layer_off = s->layer_off[L.cache_layer];
     p.out = s->olat;
+    auto it = s->groups.find(d.heads);
+    if (s->interleaved && it != s->groups.end() && lay::latent_attention_mfma_fits(d.kv_rank, d.rot_dim)) {
+        // bf16 cache rows: the matrix-core kernel; enough key splits to fill the chip when the
+        // step has few rows (decoding)
+        const int ng = it->second.first;
+        int S = 1024 / ng;
+        const int nb = d.window / 32 + 2;
+        S = std::max(1, std::min({S, nb, 64}));
+        if ((int64_t)ng * S > s->part_cap) {
+            QIE_HIP(hipStreamSynchronize(e->stream));
+            if (s->part_o) hipFree(s->part_o);
+            if (s->part_ml) hipFree(s->part_ml);
+            s->part_o = s->part_ml = nullptr;
+            s->part_cap = 0;
+            const int64_t units = ((int64_t)ng * S + 255) / 256 * 256;
+            QIE_TRY(dmalloc((void**)&s->part_o, (size_t)units * 16 * s->m_r * 4));
+            QIE_TRY(dmalloc((void**)&s->part_ml, (size_t)units * 16 * 2 * 4));
+            s->part_cap = units;
+        }
+        lay::LatentAttnMfmaP q{};
+        q.q_abs = s->qabs; q.proj = s->proj; q.ld = L.n_in;
+        q.row_slot = s->row_slot; q.row_pos = s->row_pos;
+        q.groups = s->d_groups + it->second.second;
+        q.n_groups = ng; q.S = S;
+        q.heads = d.heads; q.dim = d.dim; q.rot = d.rot_dim; q.R = d.kv_rank; q.window = d.window;
+        q.scale = d.scale;
+        q.cache = p.cache; q.layer_off = p.layer_off;
+        q.part_o = s->part_o; q.part_ml = s->part_ml; q.out = s->olat;
+        return lay::latent_attention_mfma(q, e->stream);
+    }
     return lay::latent_attention(p, m->f32, T, e->stream);
+}
+
+// Row groups of a step for the matrix-core attention, one list per distinct head count: heads
+// >= 16 split a token's heads into groups of 16; fewer heads put 16 / heads consecutive tokens of
+// one entry into a group.
+static int build_groups(qie_batch* b, int n_entries, const int32_t* counts) {
+    LayeredBatch* s = b->lb;
+    const LayeredModel* m = b->e->lm;
+    s->groups.clear();
+    s->h_groups.clear();
+    if (!s->interleaved) return 0;
+    for (const LayerDev& L : m->L) {
+        const int H = L.d.heads;
+        if (s->groups.count(H)) continue;
+        const int64_t first = (int64_t)s->h_groups.size();
+        int row = 0;
+        for (int i = 0; i < n_entries; i++) {
+            if (H >= 16) {
+                for (int k = 0; k < counts[i]; k++)
+                    for (int h0 = 0; h0 < H; h0 += 16) s->h_groups.push_back(int4{row + k, 1, h0, std::min(16, H - h0)});
+            } else {
+                const int tpg = 16 / H;
+                for (int k = 0; k < counts[i]; k += tpg) s->h_groups.push_back(int4{row + k, std::min(tpg, counts[i] - k), 0, H});
+            }
+            row += counts[i];
+        }
+        s->groups[H] = {(int)(s->h_groups.size() - first), first};
+    }
+    if ((int64_t)s->h_groups.size() > s->groups_cap) {
+        QIE_HIP(hipStreamSynchronize(b->e->stream));
+        if (s->d_groups) hipFree(s->d_groups);
+        s->d_groups = nullptr;
+        s->groups_cap = 0;
+        const int64_t cap = ((int64_t)s->h_groups.size() + 1023) / 1024 * 1024;
+        QIE_TRY(dmalloc((void**)&s->d_groups, (size_t)cap * sizeof(int4)));
+        s->groups_cap = cap;
+    }
+    QIE_HIP(hipMemcpyAsync(s->d_groups, s->h_groups.data(), s->h_groups.size() * sizeof(int4), hipMemcpyHostToDevice,
+                           b->e->stream));
+    return 0;
 }
 
 static int enq_mixer_out(qie_batch* b, int i, int T) {
@@ -622,16 +701,22 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
     b->max_pages = (max_ctx + page_tokens - 1) / page_tokens;
     b->n_pages = n_pages > 0 ? n_pages : batch * b->max_pages + 1;
     s->layer_off.assign(m->a.n_layers, 0);
+    // bf16 caches whose every layer fits the matrix-core attention carry, after the rows of a
+    // caching layer, the key-interleaved copy of c (R more elements per token)
+    s->interleaved = !m->f32;
+    for (int i = 0; i < m->a.n_layers; i++)
+        if (!lay::latent_attention_mfma_fits(m->L[i].d.kv_rank, m->L[i].d.rot_dim)) s->interleaved = false;
     int64_t off = 0;
     for (int i = 0; i < m->a.n_layers; i++) {
         const qie_layer_desc& d = m->L[i].d;
         if (d.kv_from < 0) {
             s->layer_off[i] = off;
-            off += (int64_t)page_tokens * (d.kv_rank + d.rot_dim);
+            off += (int64_t)page_tokens * (d.kv_rank + d.rot_dim + (s->interleaved ? d.kv_rank : 0));
         }
         const int64_t H = d.heads;
         s->m_in = std::max<int64_t>(s->m_in, m->L[i].n_in);
         s->m_hr = std::max<int64_t>(s->m_hr, H * d.kv_rank);
+        s->m_r = std::max<int64_t>(s->m_r, d.kv_rank);
         s->m_hv = std::max<int64_t>(s->m_hv, H * d.vdim);
         const int64_t k = d.ff_kind == QIE_FF_MOE ? d.top : 1;
         if (d.ff_kind != QIE_FF_NONE) {
@@ -673,7 +758,7 @@ void layered_batch_destroy(qie_batch* b) {
     LayeredBatch* s = b->lb;
     if (!s) return;
     lb_free(s);
-    void* ps[] = {s->want, s->xn, s->logits, s->logits_bf, s->d_ids, s->d_step};
+    void* ps[] = {s->want, s->xn, s->logits, s->logits_bf, s->d_ids, s->d_step, s->d_groups, s->part_o, s->part_ml};
     for (void* p : ps)
         if (p) hipFree(p);
     if (s->h_stage) hipHostFree(s->h_stage);
@@ -833,6 +918,7 @@ int qie_batch_step(qie_batch* b, int32_t n_entries, const int32_t* slots, const 
     QIE_HIP(hipMemcpyAsync(s->row_slot, hs, (size_t)T * 4, hipMemcpyHostToDevice, st));
     QIE_HIP(hipMemcpyAsync(s->row_pos, hs + R, (size_t)T * 4, hipMemcpyHostToDevice, st));
     QIE_HIP(hipMemcpyAsync(s->tok, hs + 2 * R, (size_t)T * 4, hipMemcpyHostToDevice, st));
+    QIE_TRY(build_groups(b, n_entries, counts));
     if (n_want > 0) QIE_HIP(hipMemcpyAsync(s->want, want_rows, (size_t)n_want * 4, hipMemcpyHostToDevice, st));
     QIE_TRY(enq_forward(b, (int)T, n_want));
     s->last_T = (int)T;

@@ -178,6 +178,14 @@ __global__ __launch_bounds__(256) void latent_post_kernel(LatentPostP p) {
     const float inv = 1.0f / sqrtf(ss / (float)p.R + p.eps);
     TC* out = (TC*)latent_row(p.cache, slot, pos, p.layer_off, p.R + p.rot, sizeof(TC));
     for (int i = tid; i < p.R; i += 256) stf<TC>(out, i, d[i] * inv * p.norm_w[i]);
+    if (p.interleaved) {
+        // second copy of c for the value product of the matrix-core attention: the 4 keys of a
+        // group side by side for every latent coordinate
+        const int pt = pos % p.cache.page_tokens;
+        TC* region = out - (int64_t)pt * (p.R + p.rot);
+        TC* ct = region + (int64_t)p.cache.page_tokens * (p.R + p.rot) + (int64_t)(pt >> 2) * p.R * 4 + (pt & 3);
+        for (int i = tid; i < p.R; i += 256) stf<TC>(ct, (int64_t)i * 4, d[i] * inv * p.norm_w[i]);
+    }
     const float* kr = d + p.R;
     for (int j = tid; j < p.rot; j += 256) {
         float v;

@@ -47,6 +47,7 @@ struct LatentPostP {
     const float* rope_sin;
     LatentCache cache;
     int64_t layer_off;
+    int interleaved;      // bf16 caches: also write the key-interleaved copy of c that follows the rows
 };
 int latent_post(const LatentPostP& p, bool cache_f32, int T, hipStream_t st);
 
@@ -63,6 +64,30 @@ struct LatentAttnP {
     float* out;           // [T][heads][R]
 };
 int latent_attention(const LatentAttnP& p, bool cache_f32, int T, hipStream_t st);
+
+// The matrix-core form (k_latent_attn.hip; bf16 cache rows followed, per caching layer and page,
+// by the key-interleaved copy of c: element ((t % page_tokens) / 4 * R + r) * 4 + t % 4).  A row
+// group is up to 16 (token, head) rows of consecutive tokens of one slot: {first packed row,
+// tokens, first head, heads per token}.  S splits over the keys; part_o [groups * S][16][R] and
+// part_ml [groups * S][16][2] are scratch.
+struct LatentAttnMfmaP {
+    const float* q_abs;
+    const float* proj;
+    int64_t ld;
+    const int32_t* row_slot;
+    const int32_t* row_pos;
+    const int4* groups;
+    int n_groups, S;
+    int heads, dim, rot, R, window;
+    float scale;
+    LatentCache cache;
+    int64_t layer_off;
+    float* part_o;
+    float* part_ml;
+    float* out;           // [T][heads][R]
+};
+bool latent_attention_mfma_fits(int R, int rot);
+int latent_attention_mfma(const LatentAttnMfmaP& p, hipStream_t st);
 
 int embed_rows(const void* E, bool w_f32, const int32_t* tok, float* out, int T, int W, int vocab, hipStream_t st);
 int head_gate(float* v, const float* proj, int64_t ld, int g_col, int heads, int vd, int T, hipStream_t st);

@@ -241,6 +241,36 @@ def test_other_sizes_wide_latent_and_many_heads(model):
     assert rel(feed(m, 0, toks, [33, 2, 20]), m.ref(toks)) < REL32
 
 
+# ------------------------------------------------------------------ bf16 engines on the matrix cores
+@pytest.mark.parametrize("heads,kv_rank,rot_dim,window", [(4, 32, 8, 21), (16, 144, 16, 40), (20, 272, 8, 33), (3, 48, 0, 37)],
+                         ids=["4h-r32", "16h-r144", "20h-r272", "3h-r48-norot"])
+def test_bf16_matrix_core_shapes(model, heads, kv_rank, rot_dim, window):
+    """Sizes that take the bf16 MFMA kernels (products through the GEMM / GEMV kernels, attention
+    on the matrix cores with the key-interleaved cache copy): whole prompts, portions and single
+    tokens against the oracle, with a peaky softmax so that a wrong edge or a lost key shows."""
+    layers = [att(heads=heads, dim=16, rot_dim=rot_dim, vdim=8, kv_rank=kv_rank, window=window, scale=0.6,
+                  mlp=("moe", 32, 4, 2)),
+              att(heads=heads, dim=16, rot_dim=rot_dim, vdim=24, kv_rank=kv_rank, window=window // 2 + 1, scale=0.6, kv_from=0,
+                  mlp=("dense", 96))]
+    m = model(layers, seed=heads + kv_rank, vocab=160, width=64, dtype="bfloat16", page_tokens=16, max_ctx=512)
+    toks = m.tokens(150)
+    want = m.ref(toks)
+    cfg2 = {**m.cfg, "layers": [{**L, "mixer": {**L["mixer"], "mask": {"size": L["mixer"]["mask"]["size"] + 1}}}
+                                for L in m.cfg["layers"]]}
+    assert rel_most(O.forward(cfg2, m.T, toks), want, 0.97) > 2 * REL16   # the oracle itself reacts to the edge
+    whole = m.batch.step([(0, toks)], range(len(toks)))
+    assert rel_most(whole, want) < REL16
+    parts = feed(m, 1, toks, [2, 45, 19, 64])                          # then 20 single tokens
+    assert rel_most(parts, want) < REL16
+    # beside another request, with a step of more than 256 routed rows (experts on the MFMA kernels)
+    other = m.tokens(140)
+    got = m.batch.step([(2, other), (3, toks[:130])], range(140 + 130))
+    assert rel_most(got[:140], m.ref(other)) < REL16
+    assert rel_most(got[140:], want[:130]) < REL16
+    rest = feed(m, 3, toks[130:], [])
+    assert rel_most(rest, want[130:]) < REL16
+
+
 # ------------------------------------------------------------------ generation through the scheduler
 def oracle_greedy(m, prompt, n):
     toks, out = list(prompt), []
