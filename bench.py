@@ -48,6 +48,14 @@ STREAM_SRC = "profiles/r05_step_floor.txt (tools/step_floor.hip)"
 METRIC = "decode tokens/s + prefill tok/s, Qwen2-7B bf16 batch=1, 1/2/4/8 MI355X"
 
 
+# Layered-model sizes of `--layered`: (width, heads, dim, rot_dim, vdim, kv_rank, window, dense ff, experts, top,
+# expert ff, vocab).  Four layers: dense, routed + borrowed cache, dense, routed + borrowed cache.
+LAYERED_SIZES = {
+    "1k": (1024, 16, 64, 32, 64, 256, 512, 2816, 8, 2, 704, 32000),
+    "2k": (2048, 16, 128, 64, 128, 512, 1024, 5632, 8, 2, 1408, 32000),
+}
+
+
 def parse(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -84,6 +92,10 @@ def parse(argv=None):
                     help="N > 1 (tensor-parallel): timed decode steps of the Qwen2-72B config-5 line")
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the other single-GPU BASELINE configs (2 and 4) in the default line")
+    ap.add_argument("--layered", choices=sorted(LAYERED_SIZES), default=None,
+                    help="instead of the default workload: prefill and decode throughput of a layered (Tivazen) "
+                         "model at this size with random weights, per-stage times, and the Qwen decoder at "
+                         "equal width / heads / ffn / layers beside it (one JSON line of its own)")
     ap.add_argument("--dry-run", action="store_true",
                     help="launcher only: print the child ranks' environments as JSON and exit (no GPU)")
     return ap.parse_args(argv)
@@ -137,7 +149,139 @@ def main(argv=None):
     if a.dry_run:
         print(json.dumps({"world": int(os.environ.get("WORLD_SIZE", "1"))}))
         return 0
+    if a.layered:
+        return run_layered(a)
     return run(a)
+
+
+def layered_model(S, size):
+    """(LayeredSpec, {name: bf16 words}) at one of LAYERED_SIZES; weights ~ N(0, 1 / fan_in) drawn from one
+    pool (values repeat across tensors: timings do not care)."""
+    W, H, dim, rot, vd, R, win, ff, E, top, eff, V = LAYERED_SIZES[size]
+    mk = lambda kv_from: S.LatentAttention(H, dim, rot, vd, R, win, rot, 10000.0, (dim + rot) ** -0.5, kv_from)
+    layers = (S.LayerSpec(mk(None), S.FeedForward("dense", ff)), S.LayerSpec(mk(0), S.FeedForward("moe", eff, E, top)),
+              S.LayerSpec(mk(None), S.FeedForward("dense", ff)), S.LayerSpec(mk(2), S.FeedForward("moe", eff, E, top)))
+    spec = S.LayeredSpec(f"tivazen-{size}", W, V, 1e-6, layers, True)
+    pool = np.random.default_rng(0).standard_normal(1 << 22).astype(np.float32)
+    tensors = {}
+    for k, (name, shape) in enumerate(spec.tensor_shapes().items()):
+        n = int(np.prod(shape)) if shape else 1
+        if name.endswith(("norm1", "norm2", "final.norm")):
+            v = np.full(shape, 1.0, np.float32)
+        elif name.endswith("dkv.norm"):
+            v = np.ones(shape, np.float32)
+        elif name.endswith("dwa"):
+            v = np.asarray([0.1] * (shape[0] - 1) + [1.0], np.float32)
+        else:
+            fan = shape[-1] if name != "embed" else 1
+            v = (np.resize(np.roll(pool, 7919 * k), n) * fan ** -0.5).reshape(shape)
+        tensors[name] = (np.ascontiguousarray(v, np.float32).view(np.uint32) >> 16).astype(np.uint16).reshape(shape)
+    return spec, tensors
+
+
+def run_layered(a):
+    """Prefill (one step of P tokens) and decode (B single-token entries a step at context ~P) of the layered
+    model, per-stage hipEvent times at both shapes, and the Qwen decoder at equal sizes."""
+    import qwen_inference_engine_amd as Q
+    from qwen_inference_engine_amd import spec as S, weights as Wt
+    W, H, dim, rot, vd, R, win, ff, E, top, eff, V = LAYERED_SIZES[a.layered]
+    P, B, steps = a.prompt, max(a.batch, 8), min(a.steps, 128)
+    max_ctx = P + steps + 80
+    spec, tensors = layered_model(S, a.layered)
+    out = {"metric": "layered_decode_tokens_per_sec", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16",
+           "data": "synthetic (random weights, random token ids)", "higher_is_better": True,
+           "config": {"model": spec.name, "sizes": dict(zip(("width", "heads", "dim", "rot_dim", "vdim", "kv_rank", "window",
+                                                             "ff", "experts", "top", "expert_ff", "vocab"),
+                                                            LAYERED_SIZES[a.layered])),
+                      "layers": 4, "prompt": P, "decode_batch": B, "decode_steps": steps}}
+    eng = Q.Engine(spec, max_ctx=max_ctx).load_tensors(tensors)
+    del tensors
+    b = eng.batch(B, max_ctx, page_tokens=64)
+    rng = np.random.default_rng(1)
+    prompts = rng.integers(0, V, size=(B, P), dtype=np.int32)
+    # prefill: slot 0 whole prompt in one step, timed (released and repeated)
+    ts = []
+    for it in range(1 + a.prefill_iters):
+        t0 = time.perf_counter()
+        b.step([(0, prompts[0])], [P - 1], fetch=False)
+        ts.append(time.perf_counter() - t0)
+        if it < a.prefill_iters:
+            b.release(0)
+    t_pf = float(np.median(ts[1:]))
+    stages = {"prefill": {}, "decode": {}}
+
+    def stage_times(tag, rows, ctx):
+        st = stages[tag]
+        st["attention_us"] = round(b.time_stage(1, 0, 10), 2)
+        st["mixer_products_us"] = round(b.time_stage(2, 0, 10), 2)
+        st["dense_ff_us"] = round(b.time_stage(3, 0, 10), 2)
+        st["routed_ff_us"] = round(b.time_stage(3, 1, 10), 2)
+        st["layer_stack_us"] = round(b.time_stage(0, 0, 5), 2)
+        keys = min(ctx, win)
+        fl_att = 2.0 * rows * H * keys * (2 * R + rot) / (2.0 if tag == "prefill" and ctx <= win else 1.0)
+        st["attention_tflops"] = round(fl_att / st["attention_us"] / 1e6, 2)
+        fl_mix = 2.0 * rows * (W * (H * (dim + rot) + R + rot + H) + H * R * (dim + vd) + W * H * vd)
+        st["mixer_products_tflops"] = round(fl_mix / st["mixer_products_us"] / 1e6, 2)
+        st["dense_ff_tflops"] = round(2.0 * rows * 3 * W * ff / st["dense_ff_us"] / 1e6, 2)
+        st["routed_ff_tflops"] = round(2.0 * rows * top * 3 * W * eff / st["routed_ff_us"] / 1e6, 2)
+        if tag == "decode":   # bytes a decode step must read: the layer's weights once, every row's window of cache rows
+            st["attention_GBps"] = round(rows * keys * (2 * R + rot) * 2 / st["attention_us"] / 1e3, 1)
+            st["dense_ff_GBps"] = round(3 * W * ff * 2 / st["dense_ff_us"] / 1e3, 1)
+            st["mixer_products_GBps"] = round((W * (H * (dim + rot) + R + rot + H) + H * R * (dim + vd) + W * H * vd) * 2
+                                              / st["mixer_products_us"] / 1e3, 1)
+    stage_times("prefill", P, P)
+    # decode: the other slots get their prompts (in 512-token portions), then B single tokens a step
+    for s_ in range(1, B):
+        for c0 in range(0, P, 512):
+            b.step([(s_, prompts[s_][c0:c0 + 512])], [], fetch=False)
+    toks = rng.integers(0, V, size=(steps + 8, B), dtype=np.int32)
+    for i in range(8):
+        b.step([(s_, [toks[i][s_]]) for s_ in range(B)], range(B), fetch=False)
+    t0 = time.perf_counter()
+    for i in range(8, 8 + steps):
+        b.step([(s_, [toks[i][s_]]) for s_ in range(B)], range(B), fetch=False)
+        b.step_sample()
+    dt = time.perf_counter() - t0
+    stage_times("decode", B, P)
+    out.update(value=round(B * steps / dt, 1), steps=steps, warmup=8, ms_per_step=round(dt * 1e3 / steps, 4),
+               prefill_tok_s=round(P / t_pf, 1), prefill_ms=round(t_pf * 1e3, 3),
+               prefill_tflops=round(spec.step_flops(P, P // 2) / t_pf / 1e12, 2), stages=stages, vs_baseline=None)
+    b.close()
+    eng.close()
+    # the closest served model at equal size: the Qwen decoder (GQA, dense SwiGLU), same bench shapes
+    qs = S.ModelSpec(f"qwen-like-{a.layered}", 4, W, H, max(1, H // 4), 128 if H * 128 <= 4 * W else 64, ff, V, False, True, False, 1e-6)
+    qe = Q.Engine(qs, max_ctx=max_ctx).init_synthetic(Wt.SynthParams(seed=0))
+    qb = qe.batch(B, max_ctx)
+    qb.prefill(0, prompts[0])
+    tq = []
+    for _ in range(a.prefill_iters):
+        qe.sync()
+        t0 = time.perf_counter()
+        qb.prefill(0, prompts[0])
+        qe.sync()
+        tq.append(time.perf_counter() - t0)
+    for s_ in range(1, B):
+        qb.prefill(s_, prompts[s_])
+    qb.decode(8, want_ids=False)
+    qe.sync()
+    t0 = time.perf_counter()
+    qb.decode(steps, want_ids=False)
+    qe.sync()
+    dq = time.perf_counter() - t0
+    kern = {}
+    for name, which in (("gate_up", 0), ("down", 1), ("qkv", 2), ("o", 3), ("attention", 5)):
+        us, by = qb.time_kernel(which, 20)
+        kern[name] = {"us": round(us, 2), "GBps": round(by / us / 1e3, 1)}
+    out["qwen_equal_size"] = {"model": f"{qs.n_layers} layers, hidden {qs.hidden}, {qs.n_heads}/{qs.n_kv_heads} heads of "
+                                       f"{qs.head_dim}, ffn {qs.ffn}",
+                              "decode_tok_s": round(B * steps / dq, 1), "ms_per_step": round(dq * 1e3 / steps, 4),
+                              "prefill_tok_s": round(P / float(np.median(tq)), 1),
+                              "prefill_tflops": round(qs.prefill_flops(P) / float(np.median(tq)) / 1e12, 2),
+                              "decode_kernels_B%d" % B: kern}
+    qb.close()
+    qe.close()
+    print(json.dumps(out), flush=True)
+    return 0
 
 
 def run(a):

@@ -293,7 +293,7 @@ static int finalize_layer(qie_engine* e, LayeredModel* m, int i) {
 // ------------------------------------------------------------------ the step
 static int lin(const qie_engine* e, const float* A, int64_t lda, const void* Wt, int64_t ldw, float* Y, int64_t ldy, int M, int N,
                int K, int batch = 1, int64_t sA = 0, int64_t sW = 0, int64_t sY = 0, const int32_t* grp = nullptr) {
-    lay::LinearP p{A, lda, Wt, ldw, Y, ldy, M, N, K, batch, sA, sW, sY, e->lm->f32 ? 0 : 1, grp};
+    lay::LinearP p{A, lda, Wt, ldw, Y, ldy, M, N, K, batch, sA, sW, sY, e->lm->f32 ? 0 : 1, grp, e->lm->f32 ? 0 : 1};
     return lay::linear(p, e->lm->f32, e->stream);
 }
 
@@ -369,20 +369,6 @@ static int enq_absorb(qie_batch* b, int i, int T) {
     LayeredBatch* s = b->lb;
     const int hq = d.dim + d.rot_dim;
     const int64_t HR = (int64_t)d.heads * d.kv_rank, HQ = (int64_t)d.heads * hq;
-    if (!e->lm->f32 && T > 16 && d.dim % 8 == 0 && hq % 8 == 0 && d.kv_rank % 4 == 0) {
-        // prompt-sized steps: one MFMA product per head on the bf16 image of the query rows
-        QIE_TRY(lay::rows_to_bf16_strided(s->proj, L.n_in, s->abf, HQ, T, (int)HQ, e->stream));
-        for (int h = 0; h < d.heads; h++) {
-            qie_linear_args a{};
-            a.x = s->abf + (int64_t)h * hq; a.ldx = HQ;
-            a.w[0] = (const uint16_t*)L.uk_t + (int64_t)h * d.kv_rank * d.dim; a.seg_rows[0] = d.kv_rank;
-            a.M = T; a.K = d.dim; a.N = d.kv_rank;
-            a.y = s->qabs + (int64_t)h * d.kv_rank; a.ldy = HR;
-            a.epilogue = QIE_EPI_F32;
-            QIE_TRY(qie_linear(&a, e->stream));
-        }
-        return 0;
-    }
     return lin(e, s->proj, L.n_in, L.uk_t, d.dim, s->qabs, HR, T, d.kv_rank, d.dim, d.heads, hq, (int64_t)d.kv_rank * d.dim,
                d.kv_rank);
 }
@@ -409,7 +395,7 @@ static int enq_attention(qie_batch* b, int i, int T) {
         // bf16 cache rows: the matrix-core kernel; enough key splits to fill the chip when the
         // step has few rows (decoding)
         const int ng = it->second.first;
-        int S = 1024 / ng;
+        int S = 1024 * lay::kLatentQG / ng;
         const int nb = d.window / 32 + 2;
         S = std::max(1, std::min({S, nb, 64}));
         if ((int64_t)ng * S > s->part_cap) {
@@ -459,6 +445,8 @@ static int build_groups(qie_batch* b, int n_entries, const int32_t* counts) {
                 const int tpg = 16 / H;
                 for (int k = 0; k < counts[i]; k += tpg) s->h_groups.push_back(int4{row + k, std::min(tpg, counts[i] - k), 0, H});
             }
+            // whole units per entry: a unit's groups share the slot
+            while ((s->h_groups.size() - first) % lay::kLatentQG) s->h_groups.push_back(int4{row, 0, 0, 1});
             row += counts[i];
         }
         s->groups[H] = {(int)(s->h_groups.size() - first), first};
@@ -485,21 +473,8 @@ static int enq_mixer_out(qie_batch* b, int i, int T) {
     LayeredBatch* s = b->lb;
     const int64_t HV = (int64_t)d.heads * d.vdim;
     const int64_t HR = (int64_t)d.heads * d.kv_rank;
-    if (!m->f32 && T > 16 && d.kv_rank % 8 == 0 && d.vdim % 4 == 0) {
-        QIE_TRY(lay::rows_to_bf16_strided(s->olat, HR, s->abf, HR, T, (int)HR, e->stream));
-        for (int h = 0; h < d.heads; h++) {
-            qie_linear_args a{};
-            a.x = s->abf + (int64_t)h * d.kv_rank; a.ldx = HR;
-            a.w[0] = (const uint16_t*)L.uv + (int64_t)h * d.vdim * d.kv_rank; a.seg_rows[0] = d.vdim;
-            a.M = T; a.K = d.kv_rank; a.N = d.vdim;
-            a.y = s->ov + (int64_t)h * d.vdim; a.ldy = HV;
-            a.epilogue = QIE_EPI_F32;
-            QIE_TRY(qie_linear(&a, e->stream));
-        }
-    } else {
-        QIE_TRY(lin(e, s->olat, HR, L.uv, d.kv_rank, s->ov, HV, T, d.vdim, d.kv_rank, d.heads, d.kv_rank,
-                    (int64_t)d.vdim * d.kv_rank, d.vdim));
-    }
+    QIE_TRY(lin(e, s->olat, HR, L.uv, d.kv_rank, s->ov, HV, T, d.vdim, d.kv_rank, d.heads, d.kv_rank, (int64_t)d.vdim * d.kv_rank,
+                d.vdim));
     QIE_TRY(lay::head_gate(s->ov, s->proj, L.n_in, L.g_col, d.heads, d.vdim, T, e->stream));
     return dense(b, s->ov, HV, L.wo, s->mix, m->a.width, T, m->a.width, (int)HV);
 }

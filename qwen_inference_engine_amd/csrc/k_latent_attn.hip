@@ -28,39 +28,52 @@ __device__ __forceinline__ const uint16_t* page_base(const LatentCache& c, int s
     return (const uint16_t*)c.pool + (int64_t)page * c.page_stride + layer_off;
 }
 
-template <int RT, int KS>
-__global__ __launch_bounds__(64) void latent_attn_mfma_kernel(LatentAttnMfmaP p) {
-    const int lane = threadIdx.x, g = lane >> 4, n = lane & 15;
-    const int unit = blockIdx.x, grp = unit / p.S, sp = unit % p.S;
-    const int4 G = p.groups[grp];   // first packed row, tokens, first head, heads per token
-    const int nrows = G.y * G.w;
-    const bool vrow = n < nrows;
-    const int tok = G.x + (vrow ? n / G.w : 0), head = G.z + (vrow ? n % G.w : 0);
-    const int slot = p.row_slot[G.x];
-    const int mypos = p.row_pos[tok];
-    const int hi = p.row_pos[G.x + G.y - 1];
-    int lo = p.row_pos[G.x] - p.window + 1;
-    if (lo < 0) lo = 0;
+// QG row groups per wave (consecutive groups of one entry: neighbouring tokens, or the head
+// groups of one token) share every loaded cache fragment; the 4 waves of a workgroup take
+// neighbouring units of the same key split, so their loads of the same rows meet in the L1.
+template <int RT, int KS, int QG>
+__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentAttnMfmaP p) {
+    const int lane = threadIdx.x & 63, g = lane >> 4, n = lane & 15;
+    const int n_units = p.n_groups / QG;
+    const int v = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (v >= n_units * p.S) return;
+    const int sp = v / n_units, unit = v % n_units;
     const int R = p.R, D = p.R + p.rot, PT = p.cache.page_tokens;
     const int nrt = R >> 4;
 
-    // this lane's query row as B fragments (bf16), zero beyond D and for unused rows
-    bf16x8_t qf[KS];
-    {
+    bool vrow[QG];
+    int mypos[QG];
+    bf16x8_t qf[QG][KS];
+    int lo = 0x7fffffff, hi = -1, slot = 0, nq = 0;
+#pragma unroll
+    for (int q = 0; q < QG; q++) {
+        const int4 G = p.groups[unit * QG + q];   // first packed row, tokens, first head, heads per token
+        vrow[q] = n < G.y * G.w;
+        const int tok = G.x + (vrow[q] ? n / G.w : 0), head = G.z + (vrow[q] ? n % G.w : 0);
+        mypos[q] = p.row_pos[tok];
+        if (G.y > 0) {
+            nq = q + 1;
+            slot = p.row_slot[G.x];
+            lo = min(lo, p.row_pos[G.x]);
+            hi = max(hi, p.row_pos[G.x + G.y - 1]);
+        }
+        // this lane's query row as B fragments (bf16), zero beyond D and for unused rows
         const float* qa = p.q_abs + ((int64_t)tok * p.heads + head) * R;
         const float* qr = p.proj + (int64_t)tok * p.ld + (int64_t)head * (p.dim + p.rot) + p.dim;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
             const int d0 = ks * 32 + 8 * g;
             uint32_t w[4] = {0u, 0u, 0u, 0u};
-            if (vrow && d0 < D) {
+            if (vrow[q] && d0 < D) {
                 const float* src = d0 < R ? qa + d0 : qr + (d0 - R);   // R and rot are multiples of 8
 #pragma unroll
                 for (int j = 0; j < 4; j++) w[j] = pack2(src[2 * j], src[2 * j + 1]);
             }
-            qf[ks] = __builtin_bit_cast(bf16x8_t, make_uint4(w[0], w[1], w[2], w[3]));
+            qf[q][ks] = __builtin_bit_cast(bf16x8_t, make_uint4(w[0], w[1], w[2], w[3]));
         }
     }
+    lo = lo - p.window + 1;
+    if (lo < 0) lo = 0;
 
     const int kb_lo = lo >> 5, kb_hi = hi >> 5;
     const int per = (kb_hi - kb_lo + 1 + p.S - 1) / p.S;
@@ -68,68 +81,84 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_kernel(LatentAttnMfmaP p)
     int b1 = b0 + per;
     if (b1 > kb_hi + 1) b1 = kb_hi + 1;
 
-    f32x4_t oacc[RT];
+    f32x4_t oacc[QG][RT];
+    float m_run[QG], l_run[QG];
 #pragma unroll
-    for (int rt = 0; rt < RT; rt++) oacc[rt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY, l_run = 0.f;
+    for (int q = 0; q < QG; q++) {
+        m_run[q] = -INFINITY;
+        l_run[q] = 0.f;
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) oacc[q][rt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
 
     for (int kb = b0; kb < b1; kb++) {
         const int k0 = kb << 5;
-        f32x4_t sacc[2];
+        f32x4_t sacc[QG][2];
 #pragma unroll
         for (int t = 0; t < 2; t++) {
-            sacc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int q = 0; q < QG; q++) sacc[q][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
             int key = k0 + 16 * t + n;
             if (key > hi) key = hi;   // masked below; keeps the address inside the slot's pages
             const uint16_t* row = page_base(p.cache, slot, key, p.layer_off) + (int64_t)(key % PT) * D;
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) {
                 const int d0 = ks * 32 + 8 * g;
-                uint4 kv = make_uint4(0u, 0u, 0u, 0u);
-                if (d0 < D) kv = *reinterpret_cast<const uint4*>(row + d0);
-                sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kv), qf[ks], sacc[t], 0, 0, 0);
+                // no branch around a load: loads inside conditional blocks are waited for one
+                // by one; beyond D the query fragment is zero, so any finite values do
+                const uint4 kv = *reinterpret_cast<const uint4*>(row + (d0 < D ? d0 : 0));
+#pragma unroll
+                for (int q = 0; q < QG; q++)
+                    sacc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kv), qf[q][ks], sacc[q][t],
+                                                                         0, 0, 0);
             }
         }
-        // scores of query row n against keys k0 + 16 t + 4 g + j
-        float sv[8];
-        float mloc = -INFINITY;
+        bf16x8_t pbh[QG], pbl[QG];
+        float alpha[QG];
 #pragma unroll
-        for (int t = 0; t < 2; t++)
+        for (int q = 0; q < QG; q++) {
+            // scores of query row n against keys k0 + 16 t + 4 g + j
+            float sv[8];
+            float mloc = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const int key = k0 + 16 * t + 4 * g + j;
+                    const bool ok = vrow[q] && key <= mypos[q] && key > mypos[q] - p.window;
+                    const float sc = ok ? sacc[q][t][j] * p.scale : -INFINITY;
+                    sv[4 * t + j] = sc;
+                    mloc = fmaxf(mloc, sc);
+                }
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+            const float m_new = fmaxf(m_run[q], mloc);
+            float pe[8];
+            alpha[q] = 1.f;
+            if (m_new == -INFINITY) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) pe[i] = 0.f;
+            } else {
+                alpha[q] = expf(m_run[q] - m_new);
+                float ls = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    pe[i] = expf(sv[i] - m_new);
+                    ls += pe[i];
+                }
+                l_run[q] = l_run[q] * alpha[q] + ls;
+                m_run[q] = m_new;
+            }
+            // P = hi + lo bf16 parts, in k-slot order
+            uint32_t ph[4], pl[4];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const int key = k0 + 16 * t + 4 * g + j;
-                const bool ok = vrow && key <= mypos && key > mypos - p.window;
-                const float s = ok ? sacc[t][j] * p.scale : -INFINITY;
-                sv[4 * t + j] = s;
-                mloc = fmaxf(mloc, s);
+                ph[j] = pack2(pe[2 * j], pe[2 * j + 1]);
+                pl[j] = pack2(pe[2 * j] - bf_lo(ph[j]), pe[2 * j + 1] - bf_hi(ph[j]));
             }
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-        const float m_new = fmaxf(m_run, mloc);
-        float alpha = 1.f, pe[8];
-        if (m_new == -INFINITY) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) pe[i] = 0.f;
-        } else {
-            alpha = expf(m_run - m_new);
-            float ls = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                pe[i] = expf(sv[i] - m_new);
-                ls += pe[i];
-            }
-            l_run = l_run * alpha + ls;
-            m_run = m_new;
+            pbh[q] = __builtin_bit_cast(bf16x8_t, make_uint4(ph[0], ph[1], ph[2], ph[3]));
+            pbl[q] = __builtin_bit_cast(bf16x8_t, make_uint4(pl[0], pl[1], pl[2], pl[3]));
         }
-        // P = hi + lo bf16 parts, in k-slot order
-        uint32_t ph[4], pl[4];
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            ph[j] = pack2(pe[2 * j], pe[2 * j + 1]);
-            pl[j] = pack2(pe[2 * j] - bf_lo(ph[j]), pe[2 * j + 1] - bf_hi(ph[j]));
-        }
-        const bf16x8_t pbh = __builtin_bit_cast(bf16x8_t, make_uint4(ph[0], ph[1], ph[2], ph[3]));
-        const bf16x8_t pbl = __builtin_bit_cast(bf16x8_t, make_uint4(pl[0], pl[1], pl[2], pl[3]));
         // key-interleaved c: element ((key % PT) / 4 * R + r) * 4 + key % 4 after the PT x D rows
         const uint16_t* ct[2];
 #pragma unroll
@@ -138,56 +167,82 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_kernel(LatentAttnMfmaP p)
             if (key4 > hi) key4 = hi & ~3;
             ct[t] = page_base(p.cache, slot, key4, p.layer_off) + (int64_t)PT * D + (int64_t)((key4 % PT) >> 2) * R * 4;
         }
+        // latent tiles in runs of 4 behind one uniform branch, the 8 loads of a run unconditional
+        // (a tile past R reads tile 0 again and its product is dropped at the end)
 #pragma unroll
-        for (int rt = 0; rt < RT; rt++) {
-            if (rt < nrt) {
-                const int r = 16 * rt + n;
-                const uint2 v0 = *reinterpret_cast<const uint2*>(ct[0] + r * 4);
-                const uint2 v1 = *reinterpret_cast<const uint2*>(ct[1] + r * 4);
-                const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(v0.x, v0.y, v1.x, v1.y));
-                oacc[rt] = oacc[rt] * alpha;
-                oacc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pbh, oacc[rt], 0, 0, 0);
-                oacc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pbl, oacc[rt], 0, 0, 0);
+        for (int rc = 0; rc < RT; rc += 4) {
+            if (rc < nrt) {
+                uint2 v0[4], v1[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int r = (rc + i < nrt ? 16 * (rc + i) : 0) + n;
+                    v0[i] = *reinterpret_cast<const uint2*>(ct[0] + r * 4);
+                    v1[i] = *reinterpret_cast<const uint2*>(ct[1] + r * 4);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(v0[i].x, v0[i].y, v1[i].x, v1[i].y));
+#pragma unroll
+                    for (int q = 0; q < QG; q++) {
+                        oacc[q][rc + i] = oacc[q][rc + i] * alpha[q];
+                        oacc[q][rc + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pbh[q], oacc[q][rc + i], 0, 0, 0);
+                        oacc[q][rc + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pbl[q], oacc[q][rc + i], 0, 0, 0);
+                    }
+                }
             }
         }
     }
-    l_run += __shfl_xor(l_run, 16, 64);
-    l_run += __shfl_xor(l_run, 32, 64);
-    if (g == 0) {
-        p.part_ml[((int64_t)unit * 16 + n) * 2] = m_run;
-        p.part_ml[((int64_t)unit * 16 + n) * 2 + 1] = l_run;
-    }
-    float* po = p.part_o + ((int64_t)unit * 16 + n) * R;
 #pragma unroll
-    for (int rt = 0; rt < RT; rt++)
-        if (rt < nrt) *reinterpret_cast<float4*>(po + 16 * rt + 4 * g) = make_float4(oacc[rt][0], oacc[rt][1], oacc[rt][2], oacc[rt][3]);
+    for (int q = 0; q < QG; q++) {
+        float l = l_run[q];
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
+        const int64_t u = (((int64_t)(unit * QG + q)) * p.S + sp) * 16 + n;
+        if (g == 0) {
+            p.part_ml[u * 2] = m_run[q];
+            p.part_ml[u * 2 + 1] = l;
+        }
+        float* po = p.part_o + u * R;
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++)
+            if (rt < nrt)
+                *reinterpret_cast<float4*>(po + 16 * rt + 4 * g) =
+                    make_float4(oacc[q][rt][0], oacc[q][rt][1], oacc[q][rt][2], oacc[q][rt][3]);
+    }
 }
 
-// merges the key splits of one row group: out[tok, head, :] = sum_s e^(m_s - M) O_s / sum_s e^(m_s - M) l_s
+// merges the key splits of one (token, head) row: out = sum_s e^(m_s - M) O_s / sum_s e^(m_s - M) l_s.
+// One block per row of a group; the split weights go through LDS so that the loads of the
+// partial outputs are independent of each other.
 __global__ __launch_bounds__(256) void latent_combine_kernel(LatentAttnMfmaP p) {
-    const int grp = blockIdx.x;
+    __shared__ float w[64];
+    __shared__ float inv_s;
+    const int grp = blockIdx.x >> 4, n = blockIdx.x & 15;
     const int4 G = p.groups[grp];
-    const int nrows = G.y * G.w, R = p.R;
-    for (int n = 0; n < nrows; n++) {
-        const int tok = G.x + n / G.w, head = G.z + n % G.w;
-        float M = -INFINITY;
-        for (int s = 0; s < p.S; s++) M = fmaxf(M, p.part_ml[(((int64_t)grp * p.S + s) * 16 + n) * 2]);
-        float L = 0.f;
-        for (int s = 0; s < p.S; s++) {
-            const float* ml = p.part_ml + (((int64_t)grp * p.S + s) * 16 + n) * 2;
-            if (ml[0] != -INFINITY) L += expf(ml[0] - M) * ml[1];
-        }
-        const float inv = 1.0f / L;
-        float* o = p.out + ((int64_t)tok * p.heads + head) * R;
-        for (int r = threadIdx.x; r < R; r += 256) {
-            float acc = 0.f;
-            for (int s = 0; s < p.S; s++) {
-                const int64_t u = ((int64_t)grp * p.S + s) * 16 + n;
-                const float m = p.part_ml[u * 2];
-                if (m != -INFINITY) acc += expf(m - M) * p.part_o[u * R + r];
-            }
-            o[r] = acc * inv;
-        }
+    if (n >= G.y * G.w) return;
+    const int tok = G.x + n / G.w, head = G.z + n % G.w, R = p.R, S = p.S;
+    const int64_t u0 = (int64_t)grp * S * 16 + n;   // unit (grp, s) row n = u0 + 16 s
+    if (threadIdx.x < 64) {
+        const int s = threadIdx.x;
+        const float m = s < S ? p.part_ml[(u0 + 16 * s) * 2] : -INFINITY;
+        const float l = s < S ? p.part_ml[(u0 + 16 * s) * 2 + 1] : 0.f;
+        float M = m;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
+        const float e = m == -INFINITY ? 0.f : expf(m - M);
+        float L = e * l;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) L += __shfl_xor(L, o, 64);
+        w[s] = e;
+        if (s == 0) inv_s = 1.0f / L;
+    }
+    __syncthreads();
+    const float inv = inv_s;
+    float* o = p.out + ((int64_t)tok * p.heads + head) * R;
+    for (int r = threadIdx.x; r < R; r += 256) {
+        float acc = 0.f;
+        for (int s = 0; s < S; s++) acc = fmaf(w[s], p.part_o[(u0 + 16 * s) * R + r], acc);
+        o[r] = acc * inv;
     }
 }
 
@@ -197,18 +252,20 @@ bool latent_attention_mfma_fits(int R, int rot) {
 
 int latent_attention_mfma(const LatentAttnMfmaP& p, hipStream_t st) {
     QIE_REQUIRE(latent_attention_mfma_fits(p.R, p.rot), "latent attention (MFMA): latent %d + rotated %d not covered", p.R, p.rot);
-    QIE_REQUIRE(p.n_groups > 0 && p.S > 0 && p.groups && p.part_o && p.part_ml, "latent attention (MFMA): bad arguments");
+    QIE_REQUIRE(p.n_groups > 0 && p.S > 0 && p.S <= 64 && p.groups && p.part_o && p.part_ml, "latent attention (MFMA): bad arguments");
     QIE_REQUIRE(p.cache.page_tokens % 16 == 0, "latent attention (MFMA): pages of %d tokens", p.cache.page_tokens);
-    const dim3 grid((unsigned)(p.n_groups * p.S)), block(64);
+    QIE_REQUIRE(p.n_groups % kLatentQG == 0, "latent attention (MFMA): %d groups are not whole units of %d", p.n_groups, kLatentQG);
     const int D = p.R + p.rot;
+    const int waves = p.n_groups / kLatentQG * p.S;
+    const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
     if (p.R <= 128 && D <= 160)
-        hipLaunchKernelGGL((latent_attn_mfma_kernel<8, 5>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((latent_attn_mfma_kernel<8, 5, kLatentQG>), grid, block, 0, st, p);
     else if (p.R <= 256 && D <= 320)
-        hipLaunchKernelGGL((latent_attn_mfma_kernel<16, 10>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((latent_attn_mfma_kernel<16, 10, kLatentQG>), grid, block, 0, st, p);
     else
-        hipLaunchKernelGGL((latent_attn_mfma_kernel<32, 18>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((latent_attn_mfma_kernel<32, 18, kLatentQG>), grid, block, 0, st, p);
     QIE_LAUNCH_CHECK();
-    hipLaunchKernelGGL(latent_combine_kernel, dim3(p.n_groups), dim3(256), 0, st, p);
+    hipLaunchKernelGGL(latent_combine_kernel, dim3(p.n_groups * 16), dim3(256), 0, st, p);
     QIE_LAUNCH_CHECK();
     return 0;
 }

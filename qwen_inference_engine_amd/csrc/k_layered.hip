@@ -114,8 +114,153 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearP p) {
     }
 }
 
+// Few rows (decoding, or few rows per expert): one wave per output column streams the weight
+// row once with 16-byte loads and keeps up to 16 rows' sums in registers, so the launch is as
+// wide as N x batch whatever M is.  VEC: K, the row strides and the batch strides keep every
+// 8-element run aligned; else one element per lane and step.
+template <typename TW, bool VEC>
+__global__ __launch_bounds__(256) void linear_skinny_kernel(LinearP p) {
+    const int z = blockIdx.z, lane = threadIdx.x & 63;
+    const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+    int m_lo = 0, m_hi = p.M;
+    if (p.grp_off) {
+        m_lo = p.grp_off[z];
+        m_hi = p.grp_off[z + 1];
+    }
+    const int m0 = m_lo + blockIdx.y * 16;
+    if (m0 >= m_hi || n >= p.N) return;
+    const int rows = min(16, m_hi - m0);
+    const float* A = p.A + (int64_t)z * p.sA + (int64_t)m0 * p.lda;
+    const TW* W = (const TW*)p.W + (int64_t)z * p.sW + (int64_t)n * p.ldw;
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] = 0.f;
+    if (VEC) {
+        for (int k = lane * 8; k < p.K; k += 512) {
+            float w[8];
+            if (sizeof(TW) == 2) {
+                const uint4 u = *reinterpret_cast<const uint4*>((const uint16_t*)W + k);
+                w[0] = bf_lo(u.x); w[1] = bf_hi(u.x); w[2] = bf_lo(u.y); w[3] = bf_hi(u.y);
+                w[4] = bf_lo(u.z); w[5] = bf_hi(u.z); w[6] = bf_lo(u.w); w[7] = bf_hi(u.w);
+            } else {
+                const float4 u0 = *reinterpret_cast<const float4*>((const float*)W + k);
+                const float4 u1 = *reinterpret_cast<const float4*>((const float*)W + k + 4);
+                w[0] = u0.x; w[1] = u0.y; w[2] = u0.z; w[3] = u0.w; w[4] = u1.x; w[5] = u1.y; w[6] = u1.z; w[7] = u1.w;
+            }
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                if (i < rows) {
+                    const float4 a0 = *reinterpret_cast<const float4*>(A + (int64_t)i * p.lda + k);
+                    const float4 a1 = *reinterpret_cast<const float4*>(A + (int64_t)i * p.lda + k + 4);
+                    float a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+                    float t = 0.f;
+#pragma unroll
+                    for (int j = 0; j < 8; j++) t = fmaf(p.round_a ? rbf(a[j]) : a[j], w[j], t);
+                    acc[i] += t;
+                }
+            }
+        }
+    } else {
+        for (int k = lane; k < p.K; k += 64) {
+            const float w = ldf<TW>(W, k);
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+                if (i < rows) {
+                    const float a = A[(int64_t)i * p.lda + k];
+                    acc[i] = fmaf(p.round_a ? rbf(a) : a, w, acc[i]);
+                }
+        }
+    }
+    float* Y = p.Y + (int64_t)z * p.sY + (int64_t)m0 * p.ldy + n;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const float v = wave_sum(acc[i]);
+        if (lane == 0 && i < rows) Y[(int64_t)i * p.ldy] = v;
+    }
+}
+
+// Many rows, bf16 weights, batched (per head) or grouped (per expert): MFMA tiles straight from
+// memory.  A wave owns 16 rows x 64 columns; per 32 k it converts its A rows (fp32, 8 per lane)
+// to one bf16 fragment and multiplies it with 4 weight fragments (16 bytes per lane each, the
+// rows of W are the columns of the product).  The 4 waves of a workgroup take 64 rows against
+// the same columns, so the weight fragments meet in the L1.  K a multiple of 8; k beyond K has a
+// zero A fragment; rows / columns beyond the range read a valid row again and are not stored.
+typedef __bf16 lbf16x8_t __attribute__((ext_vector_type(8)));
+typedef float lf32x4_t __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void linear_mfma_kernel(LinearP p) {
+    const int z = blockIdx.z, lane = threadIdx.x & 63, g = lane >> 4, n = lane & 15;
+    int m_lo = 0, m_hi = p.M;
+    if (p.grp_off) {
+        m_lo = p.grp_off[z];
+        m_hi = p.grp_off[z + 1];
+    }
+    const int m0 = m_lo + blockIdx.y * 64 + (threadIdx.x >> 6) * 16;
+    if (m0 >= m_hi) return;
+    const int n0 = blockIdx.x * 64;
+    const int mr = min(m0 + n, m_hi - 1);
+    const float* A = p.A + (int64_t)z * p.sA + (int64_t)mr * p.lda;
+    const uint16_t* W = (const uint16_t*)p.W + (int64_t)z * p.sW;
+    const uint16_t* wr[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) wr[c] = W + (int64_t)min(n0 + 16 * c + n, p.N - 1) * p.ldw;
+    lf32x4_t acc[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) acc[c] = lf32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < p.K; k0 += 32) {
+        const int k = k0 + 8 * g;
+        const bool in = k < p.K;
+        const int kc = in ? k : 0;
+        const float4 a0 = *reinterpret_cast<const float4*>(A + kc);
+        const float4 a1 = *reinterpret_cast<const float4*>(A + kc + 4);
+        uint4 wv[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) wv[c] = *reinterpret_cast<const uint4*>(wr[c] + kc);
+        uint4 af = make_uint4(pack2(a0.x, a0.y), pack2(a0.z, a0.w), pack2(a1.x, a1.y), pack2(a1.z, a1.w));
+        if (!in) af = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+            acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lbf16x8_t, af), __builtin_bit_cast(lbf16x8_t, wv[c]),
+                                                             acc[c], 0, 0, 0);
+    }
+    // lane holds rows m0 + 4 g + j, column n0 + 16 c + n
+    float* Y = p.Y + (int64_t)z * p.sY;
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const int col = n0 + 16 * c + n;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int m = m0 + 4 * g + j;
+            if (m < m_hi && col < p.N) Y[(int64_t)m * p.ldy + col] = acc[c][j];
+        }
+    }
+}
+
+static bool al16p(const void* q) { return ((uintptr_t)q & 15) == 0; }
+
 int linear(const LinearP& p, bool w_f32, hipStream_t st) {
     QIE_REQUIRE(p.A && p.W && p.Y && p.M > 0 && p.N > 0 && p.K > 0 && p.batch > 0, "layered linear: bad arguments");
+    const int esz = w_f32 ? 4 : 2;
+    const bool a_vec = p.lda % 4 == 0 && p.sA % 4 == 0 && al16p(p.A);
+    if (p.M <= 32) {
+        const bool vec = a_vec && p.K % 8 == 0 && p.ldw % 8 == 0 && p.sW % 8 == 0 && al16p(p.W);
+        dim3 grid((unsigned)((p.N + 3) / 4), (unsigned)((p.M + 15) / 16), (unsigned)p.batch);
+        if (w_f32) {
+            if (vec) hipLaunchKernelGGL((linear_skinny_kernel<float, true>), grid, dim3(256), 0, st, p);
+            else hipLaunchKernelGGL((linear_skinny_kernel<float, false>), grid, dim3(256), 0, st, p);
+        } else {
+            if (vec) hipLaunchKernelGGL((linear_skinny_kernel<uint16_t, true>), grid, dim3(256), 0, st, p);
+            else hipLaunchKernelGGL((linear_skinny_kernel<uint16_t, false>), grid, dim3(256), 0, st, p);
+        }
+        QIE_LAUNCH_CHECK();
+        return 0;
+    }
+    if (!w_f32 && p.round_a && p.mfma && a_vec && p.K % 8 == 0 && p.ldw % 8 == 0 && p.sW % 8 == 0 && al16p(p.W)) {
+        dim3 grid((unsigned)((p.N + 63) / 64), (unsigned)((p.M + 63) / 64), (unsigned)p.batch);
+        hipLaunchKernelGGL(linear_mfma_kernel, grid, dim3(256), 0, st, p);
+        QIE_LAUNCH_CHECK();
+        return 0;
+    }
+    (void)esz;
     dim3 grid((unsigned)((p.N + LBN - 1) / LBN), (unsigned)((p.M + LBM - 1) / LBM), (unsigned)p.batch);
     if (w_f32)
         hipLaunchKernelGGL(linear_kernel<float>, grid, dim3(256), 0, st, p);

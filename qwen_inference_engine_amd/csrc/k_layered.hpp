@@ -10,7 +10,9 @@ namespace lay {
 // y[m, n] = sum_k A[m, k] W[n, k] (+ batch z: A + z sA, W + z sW, Y + z sY).  A fp32, rounded to
 // bf16 on load when round_a; W fp32 or bf16 words; Y fp32.  grp_off (device, batch + 1 entries):
 // batch z covers rows [grp_off[z], grp_off[z + 1]) of A and Y (M is then the largest row count a
-// group can have); the k loop of an element is the same whatever else the launch holds.
+// group can have).  Three kernels by shape: up to 32 rows a column-per-wave kernel, many rows of a
+// bf16 model (mfma) MFMA tiles from memory, else 64 x 64 fp32 tiles through LDS; an element's sum
+// never depends on what else the launch holds, only on which of the three ran.
 struct LinearP {
     const float* A;
     int64_t lda;
@@ -22,6 +24,7 @@ struct LinearP {
     int64_t sA, sW, sY;
     int round_a;
     const int32_t* grp_off;
+    int mfma;   // bf16 weights, many rows: the direct MFMA kernel may take the product (batched / grouped forms)
 };
 int linear(const LinearP& p, bool w_f32, hipStream_t st);
 
@@ -86,6 +89,10 @@ struct LatentAttnMfmaP {
     float* part_ml;
     float* out;           // [T][heads][R]
 };
+// Row groups a wave takes together: the group list of a step holds, per entry, a multiple of
+// kLatentQG groups (padded with empty groups {row, 0, 0, 1}), and consecutive groups of a unit
+// belong to one slot.
+constexpr int kLatentQG = 1;   // 2 measured slower at kv_rank 256 (one wave per SIMD), and spills at 512
 bool latent_attention_mfma_fits(int R, int rot);
 int latent_attention_mfma(const LatentAttnMfmaP& p, hipStream_t st);
 

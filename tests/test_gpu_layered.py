@@ -144,7 +144,8 @@ def test_whole_prompt_portions_and_decoding_agree(model, dtype):
     parts = feed(m, 2, toks, [2, 3, 11, 2, 17, 16, 2, 30])
     assert err(parts, want) < m.tol
     # the same position must not depend on the cut beyond rounding
-    bound = 1e-5 if dtype == "float32" else 2e-2
+    # (few rows and many rows take kernels that sum in different orders)
+    bound = 5e-5 if dtype == "float32" else 2e-2
     assert err(single, whole) < bound and err(parts, whole) < bound
 
 
