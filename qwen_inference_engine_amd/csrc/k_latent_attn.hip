@@ -91,16 +91,31 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentAttnMfmaP p
         for (int rt = 0; rt < RT; rt++) oacc[q][rt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
 
+    // page ids of the two 16-key tiles of a block (a tile never straddles a page), looked up one
+    // block ahead so that no cache row load waits for a table load; keys past `hi` read row `hi`
+    const int32_t* trow = p.cache.table + (int64_t)slot * p.cache.max_pages;
+    const uint16_t* pool = (const uint16_t*)p.cache.pool + p.layer_off;
+    const int pg_hi = hi >= 0 ? trow[hi / PT] : 0;
+    int pgn[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++) pgn[t] = b0 < b1 ? trow[min((b0 << 5) + 16 * t, hi) / PT] : 0;
     for (int kb = b0; kb < b1; kb++) {
         const int k0 = kb << 5;
+        int pg[2];
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            pg[t] = pgn[t];
+            pgn[t] = trow[min(k0 + 32 + 16 * t, hi) / PT];
+        }
         f32x4_t sacc[QG][2];
 #pragma unroll
         for (int t = 0; t < 2; t++) {
 #pragma unroll
             for (int q = 0; q < QG; q++) sacc[q][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
             int key = k0 + 16 * t + n;
-            if (key > hi) key = hi;   // masked below; keeps the address inside the slot's pages
-            const uint16_t* row = page_base(p.cache, slot, key, p.layer_off) + (int64_t)(key % PT) * D;
+            const bool past = key > hi;   // masked below; keeps the address inside the slot's pages
+            if (past) key = hi;
+            const uint16_t* row = pool + (int64_t)(past ? pg_hi : pg[t]) * p.cache.page_stride + (int64_t)(key % PT) * D;
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) {
                 const int d0 = ks * 32 + 8 * g;
@@ -133,22 +148,19 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentAttnMfmaP p
             mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
             mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
             const float m_new = fmaxf(m_run[q], mloc);
+            // branch-free (a branch here would fence the value loads below): while every key so
+            // far is masked the reference max is 0, all weights and the rescale factor are 0
             float pe[8];
-            alpha[q] = 1.f;
-            if (m_new == -INFINITY) {
+            const float m_ref = m_new == -INFINITY ? 0.f : m_new;
+            alpha[q] = expf(m_run[q] - m_ref);
+            float ls = 0.f;
 #pragma unroll
-                for (int i = 0; i < 8; i++) pe[i] = 0.f;
-            } else {
-                alpha[q] = expf(m_run[q] - m_new);
-                float ls = 0.f;
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    pe[i] = expf(sv[i] - m_new);
-                    ls += pe[i];
-                }
-                l_run[q] = l_run[q] * alpha[q] + ls;
-                m_run[q] = m_new;
+            for (int i = 0; i < 8; i++) {
+                pe[i] = expf(sv[i] - m_ref);
+                ls += pe[i];
             }
+            l_run[q] = l_run[q] * alpha[q] + ls;
+            m_run[q] = m_new;
             // P = hi + lo bf16 parts, in k-slot order
             uint32_t ph[4], pl[4];
 #pragma unroll
@@ -164,8 +176,10 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentAttnMfmaP p
 #pragma unroll
         for (int t = 0; t < 2; t++) {
             int key4 = k0 + 16 * t + 4 * g;
-            if (key4 > hi) key4 = hi & ~3;
-            ct[t] = page_base(p.cache, slot, key4, p.layer_off) + (int64_t)PT * D + (int64_t)((key4 % PT) >> 2) * R * 4;
+            const bool past = key4 > hi;
+            if (past) key4 = hi & ~3;
+            ct[t] = pool + (int64_t)(past ? pg_hi : pg[t]) * p.cache.page_stride + (int64_t)PT * D +
+                    (int64_t)((key4 % PT) >> 2) * R * 4;
         }
         // latent tiles in runs of 4 behind one uniform branch, the 8 loads of a run unconditional
         // (a tile past R reads tile 0 again and its product is dropped at the end)
