@@ -304,3 +304,68 @@ def test_greedy_generation_through_the_batcher(model):
             lg = m.ref(list(p) + want[:k])[-1]
             assert abs(lg[got[k]] - lg[want[k]]) < 1e-4 * np.std(lg), (rid, k)
     assert cb.batch.page_stats()[0] == 8
+
+
+# ------------------------------------------------------------------ the command-line programs
+def write_model_dir(path, cfg, T):
+    """config.json + model.safetensors (8-byte header length, JSON header, bf16 data)."""
+    import json
+    import struct
+    hdr, blob = {}, b""
+    for name, v in T.items():
+        raw = words(v).tobytes()
+        hdr[name] = {"dtype": "BF16", "shape": list(np.shape(v)), "data_offsets": [len(blob), len(blob) + len(raw)]}
+        blob += raw
+    hj = json.dumps(hdr).encode()
+    (path / "config.json").write_text(json.dumps(cfg))
+    (path / "model.safetensors").write_bytes(struct.pack("<Q", len(hj)) + hj + blob)
+
+
+def test_trace_replay_and_generate_programs(tmp_path):
+    """bin/trace_run replays interleaved requests (portions beside single tokens, a slot and its
+    pages used again) and writes the wanted logits; bin/qie generates greedily: both equal the oracle."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    rng = np.random.default_rng(81)
+    cfg, T = O.random_model(rng, vocab=89, width=40, layers=MIXED)
+    write_model_dir(tmp_path, cfg, T)
+    reqs = {k: [int(t) for t in rng.integers(0, 89, n)] for k, n in (("a", 70), ("b", 9), ("c", 33), ("d", 50), ("e", 64))}
+    want = {k: O.forward(cfg, T, v) for k, v in reqs.items()}
+    plan = [[("a", 0, 40), ("b", 0, 9)], [("a", 40, 2), ("c", 0, 33), ("d", 0, 17)], [("a", 42, 1), ("d", 17, 33)],
+            [("a", 43, 27), ("e", 0, 64)]]            # 'e' takes the slot and pages that 'b' or 'c' gave back
+    last = {k: max(p[1] + p[2] for st in plan for p in st if p[0] == k) for k in reqs}
+    lines, rows = [], []
+    for n, st in enumerate(plan):
+        entries, end, r = [], [], []
+        for k, lo, cnt in st:
+            w = list(range(0, cnt, 3)) + ([cnt - 1] if (cnt - 1) % 3 else [])
+            entries.append({"id": k, "tokens": reqs[k][lo:lo + cnt], "want": w})
+            r += [(k, lo + i) for i in w]
+            if lo + cnt == last[k]:
+                end.append(k)
+        lines.append(json.dumps({"step": n, "entries": entries, "end": end}))
+        rows.append(r)
+    lines.insert(2, json.dumps({"step": 77, "entries": [], "end": []}))      # a step that brings nothing
+    for dtype, tol, err in (("float32", REL32, rel), ("bfloat16", REL16, rel_most)):
+        out = tmp_path / ("out_" + dtype)
+        r = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", str(tmp_path), "--dtype", dtype, "--out", str(out),
+                            "--max-tokens", "256"], input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=300)
+        assert r.returncode == 0, r.stderr[-2000:]
+        assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 77", "done 2", "done 3"]
+        for n, rr in enumerate(rows):
+            got = np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(len(rr), 89)
+            ref = np.stack([want[k][i] for k, i in rr])
+            assert err(got, ref) < tol, (dtype, n)
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "qie"), "--model", str(tmp_path), "--dtype", "float32", "--gen", "5",
+                        "--prompt", ",".join(map(str, reqs["b"])), "--prompt", " ".join(map(str, reqs["c"])), "--slots", "2",
+                        "--chunk-tokens", "16"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    got = {l.split(":")[0]: [int(t) for t in l.split(":")[1].split()] for l in r.stdout.splitlines() if l.startswith("tokens[")}
+
+    class M:
+        ref = staticmethod(lambda toks: O.forward(cfg, T, toks))
+    assert got["tokens[0]"] == oracle_greedy(M, reqs["b"], 5)
+    assert got["tokens[1]"] == oracle_greedy(M, reqs["c"], 5)
