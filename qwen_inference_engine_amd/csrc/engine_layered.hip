@@ -432,6 +432,7 @@ static int build_groups(qie_batch* b, int n_entries, const int32_t* counts) {
     s->groups.clear();
     s->h_groups.clear();
     if (!s->interleaved) return 0;
+    const int pad = lay::kLatentQG;
     for (const LayerDev& L : m->L) {
         const int H = L.d.heads;
         if (s->groups.count(H)) continue;
@@ -446,7 +447,7 @@ static int build_groups(qie_batch* b, int n_entries, const int32_t* counts) {
                 for (int k = 0; k < counts[i]; k += tpg) s->h_groups.push_back(int4{row + k, std::min(tpg, counts[i] - k), 0, H});
             }
             // whole units per entry: a unit's groups share the slot
-            while ((s->h_groups.size() - first) % lay::kLatentQG) s->h_groups.push_back(int4{row, 0, 0, 1});
+            while ((s->h_groups.size() - first) % pad) s->h_groups.push_back(int4{row, 0, 0, 1});
             row += counts[i];
         }
         s->groups[H] = {(int)(s->h_groups.size() - first), first};

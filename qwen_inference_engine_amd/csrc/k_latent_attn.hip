@@ -31,8 +31,8 @@ __device__ __forceinline__ const uint16_t* page_base(const LatentCache& c, int s
 // QG row groups per wave (consecutive groups of one entry: neighbouring tokens, or the head
 // groups of one token) share every loaded cache fragment; the 4 waves of a workgroup take
 // neighbouring units of the same key split, so their loads of the same rows meet in the L1.
-template <int RT, int KS, int QG>
-__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentAttnMfmaP p) {
+template <int RT, int KS, int QG, int MINB>
+__global__ __launch_bounds__(256, MINB) void latent_attn_mfma_kernel(LatentAttnMfmaP p) {
     const int lane = threadIdx.x & 63, g = lane >> 4, n = lane & 15;
     const int n_units = p.n_groups / QG;
     const int v = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -181,29 +181,36 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentAttnMfmaP p
             ct[t] = pool + (int64_t)(past ? pg_hi : pg[t]) * p.cache.page_stride + (int64_t)PT * D +
                     (int64_t)((key4 % PT) >> 2) * R * 4;
         }
-        // latent tiles in runs of 4 behind one uniform branch, the 8 loads of a run unconditional
-        // (a tile past R reads tile 0 again and its product is dropped at the end)
+        // Value product.  A latent size that fills the instantiation (the usual case) runs all
+        // tiles with no branch in between, so the loads of the whole block are in flight together;
+        // otherwise runs of 4 tiles behind one uniform branch each (a tile past R reads tile 0
+        // again and its product is dropped at the end).
+        auto pv_run = [&](const int rc, const int cnt) {
+            uint2 v0[4], v1[4];
 #pragma unroll
-        for (int rc = 0; rc < RT; rc += 4) {
-            if (rc < nrt) {
-                uint2 v0[4], v1[4];
+            for (int i = 0; i < 4; i++) {
+                const int r = (rc + i < cnt ? 16 * (rc + i) : 0) + n;
+                v0[i] = *reinterpret_cast<const uint2*>(ct[0] + r * 4);
+                v1[i] = *reinterpret_cast<const uint2*>(ct[1] + r * 4);
+            }
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int r = (rc + i < nrt ? 16 * (rc + i) : 0) + n;
-                    v0[i] = *reinterpret_cast<const uint2*>(ct[0] + r * 4);
-                    v1[i] = *reinterpret_cast<const uint2*>(ct[1] + r * 4);
-                }
+            for (int i = 0; i < 4; i++) {
+                const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(v0[i].x, v0[i].y, v1[i].x, v1[i].y));
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, make_uint4(v0[i].x, v0[i].y, v1[i].x, v1[i].y));
-#pragma unroll
-                    for (int q = 0; q < QG; q++) {
-                        oacc[q][rc + i] = oacc[q][rc + i] * alpha[q];
-                        oacc[q][rc + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pbh[q], oacc[q][rc + i], 0, 0, 0);
-                        oacc[q][rc + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pbl[q], oacc[q][rc + i], 0, 0, 0);
-                    }
+                for (int q = 0; q < QG; q++) {
+                    oacc[q][rc + i] = oacc[q][rc + i] * alpha[q];
+                    oacc[q][rc + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pbh[q], oacc[q][rc + i], 0, 0, 0);
+                    oacc[q][rc + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pbl[q], oacc[q][rc + i], 0, 0, 0);
                 }
             }
+        };
+        if (nrt == RT) {
+#pragma unroll
+            for (int rc = 0; rc < RT; rc += 4) pv_run(rc, RT);
+        } else {
+#pragma unroll
+            for (int rc = 0; rc < RT; rc += 4)
+                if (rc < nrt) pv_run(rc, nrt);
         }
     }
 #pragma unroll
@@ -273,11 +280,11 @@ int latent_attention_mfma(const LatentAttnMfmaP& p, hipStream_t st) {
     const int waves = p.n_groups / kLatentQG * p.S;
     const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
     if (p.R <= 128 && D <= 160)
-        hipLaunchKernelGGL((latent_attn_mfma_kernel<8, 5, kLatentQG>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((latent_attn_mfma_kernel<8, 5, kLatentQG, 2>), grid, block, 0, st, p);
     else if (p.R <= 256 && D <= 320)
-        hipLaunchKernelGGL((latent_attn_mfma_kernel<16, 10, kLatentQG>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((latent_attn_mfma_kernel<16, 10, kLatentQG, 2>), grid, block, 0, st, p);
     else
-        hipLaunchKernelGGL((latent_attn_mfma_kernel<32, 18, kLatentQG>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((latent_attn_mfma_kernel<32, 18, kLatentQG, 1>), grid, block, 0, st, p);
     QIE_LAUNCH_CHECK();
     hipLaunchKernelGGL(latent_combine_kernel, dim3(p.n_groups * 16), dim3(256), 0, st, p);
     QIE_LAUNCH_CHECK();

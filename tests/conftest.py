@@ -15,6 +15,17 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "slow: long-running")
 
 
+def pytest_collection_modifyitems(config, items):
+    """The layered-engine GPU tests run after every other module.  tests/test_gpu_tp.py drives two
+    in-process ranks whose exchange kernels wait for each other: that needs the two ranks' streams
+    on different hardware queues, and which queue a new stream gets depends on how many streams the
+    process has created before.  Those tests were written under the stream history of the modules
+    before them; modules that create many engines of their own therefore go last."""
+    late = [it for it in items if "test_gpu_layered" in it.nodeid]
+    if late:
+        items[:] = [it for it in items if "test_gpu_layered" not in it.nodeid] + late
+
+
 @pytest.fixture(scope="session")
 def oracle():
     import oracle as O
