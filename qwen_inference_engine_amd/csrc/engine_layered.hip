@@ -79,7 +79,10 @@ struct LayeredBatch {
           *y = nullptr, *gu = nullptr, *act = nullptr, *ffo = nullptr, *xg = nullptr, *yd = nullptr, *score = nullptr,
           *xn = nullptr, *logits = nullptr, *keep = nullptr;
     uint16_t* logits_bf = nullptr;
-    uint16_t* abf = nullptr;      // bf16 image of a product's left operand (bf16 engines: the MFMA / GEMV kernels read bf16)
+    // bf16 engines: images written by the producing kernels (layer input, post-mixer stream, gated
+    // head outputs, activations, gathered expert rows, normed output rows)
+    uint16_t *x_bf = nullptr, *y_bf = nullptr, *ov_bf = nullptr, *act_bf = nullptr, *xg_bf = nullptr, *xn_bf = nullptr;
+    uint16_t* abf = nullptr;      // bf16 image of a product's left operand, where no producer wrote one (bf16 engines: the MFMA / GEMV kernels read bf16)
     int64_t m_abf = 0;            // its elements per row
     // matrix-core attention: row groups per head count, key-split partials
     std::map<int, std::pair<int, int64_t>> groups;   // heads -> (group count, offset into d_groups) of this step
@@ -323,7 +326,10 @@ static int dense_on(qie_batch* b, uint16_t* abf, bool staged, const float* A, in
     }
     return lin(e, A, lda, Wt, K, Y, ldy, M, N, K);
 }
-static int dense(qie_batch* b, const float* A, int64_t lda, const void* Wt, float* Y, int64_t ldy, int M, int N, int K) {
+// pre: the bf16 image of A (row stride K) when its producer wrote one
+static int dense(qie_batch* b, const float* A, int64_t lda, const void* Wt, float* Y, int64_t ldy, int M, int N, int K,
+                 const uint16_t* pre = nullptr) {
+    if (pre && lda == K) return dense_on(b, const_cast<uint16_t*>(pre), true, A, lda, Wt, Y, ldy, M, N, K);
     return dense_on(b, b->lb->abf, false, A, lda, Wt, Y, ldy, M, N, K);
 }
 
@@ -331,12 +337,12 @@ static lay::LatentCache cache_of(const qie_batch* b) {
     return lay::LatentCache{b->kc, b->seq_stride, b->d_table, b->page_tokens, b->max_pages};
 }
 
-static int enq_input_proj(qie_batch* b, int i, const float* xin, int T) {
+static int enq_input_proj(qie_batch* b, int i, const float* xin, int T, const uint16_t* xin_bf = nullptr) {
     const qie_engine* e = b->e;
     const LayeredModel* m = e->lm;
     const LayerDev& L = m->L[i];
     LayeredBatch* s = b->lb;
-    return dense(b, xin, m->a.width, L.w_in, s->proj, L.n_in, T, L.n_in, m->a.width);
+    return dense(b, xin, m->a.width, L.w_in, s->proj, L.n_in, T, L.n_in, m->a.width, xin_bf);
 }
 
 static int enq_latent_post(qie_batch* b, int i, int T) {
@@ -476,8 +482,8 @@ static int enq_mixer_out(qie_batch* b, int i, int T) {
     const int64_t HR = (int64_t)d.heads * d.kv_rank;
     QIE_TRY(lin(e, s->olat, HR, L.uv, d.kv_rank, s->ov, HV, T, d.vdim, d.kv_rank, d.heads, d.kv_rank, (int64_t)d.vdim * d.kv_rank,
                 d.vdim));
-    QIE_TRY(lay::head_gate(s->ov, s->proj, L.n_in, L.g_col, d.heads, d.vdim, T, e->stream));
-    return dense(b, s->ov, HV, L.wo, s->mix, m->a.width, T, m->a.width, (int)HV);
+    QIE_TRY(lay::head_gate(s->ov, s->ov_bf, s->proj, L.n_in, L.g_col, d.heads, d.vdim, T, e->stream));
+    return dense(b, s->ov, HV, L.wo, s->mix, m->a.width, T, m->a.width, (int)HV, s->ov_bf);
 }
 
 // feed-forward of layer i on rows y -> ffo
@@ -490,45 +496,45 @@ static int enq_ff(qie_batch* b, int i, int T) {
     const int W = m->a.width, ff = d.ff;
     hipStream_t st = e->stream;
     if (d.ff_kind == QIE_FF_DENSE) {
-        QIE_TRY(dense(b, s->y, W, L.w_gu, s->gu, 2 * ff, T, 2 * ff, W));
-        QIE_TRY(lay::silu_mul(s->gu, s->act, T, ff, st));
-        return dense(b, s->act, ff, L.w_down, s->ffo, W, T, W, ff);
+        QIE_TRY(dense(b, s->y, W, L.w_gu, s->gu, 2 * ff, T, 2 * ff, W, s->y_bf));
+        QIE_TRY(lay::silu_mul(s->gu, s->act, s->act_bf, T, ff, st));
+        return dense(b, s->act, ff, L.w_down, s->ffo, W, T, W, ff, s->act_bf);
     }
     const int E = d.experts, top = d.top, n = T * top;
     QIE_TRY(lay::route_sigmoid_topk(s->y, L.w_router, m->f32, T, W, E, top, s->sel, s->score, st));
     QIE_TRY(lay::moe_group(s->sel, n, E, s->cnt, s->off, s->slot_of, st));
-    QIE_TRY(lay::moe_gather(s->y, s->score, s->slot_of, T, top, W, s->xg, st));
-    if (!m->f32 && n >= kMoeSyncRows && W % 8 == 0 && ff % 8 == 0) {
+    const bool per_expert = !m->f32 && n >= kMoeSyncRows && W % 8 == 0 && ff % 8 == 0;
+    QIE_TRY(lay::moe_gather(s->y, s->score, s->slot_of, T, top, W, s->xg, per_expert ? s->xg_bf : nullptr, st));
+    if (per_expert) {
         // prompt-sized steps: the expert row ranges come to the host and every expert's rows go
         // through the MFMA kernels; the products are the grouped kernel's, in another order
         s->h_off.resize(E + 1);
         QIE_HIP(hipMemcpyAsync(s->h_off.data(), s->off, (size_t)(E + 1) * 4, hipMemcpyDeviceToHost, st));
         QIE_HIP(hipStreamSynchronize(st));
-        QIE_TRY(lay::rows_to_bf16_strided(s->xg, W, s->abf, W, n, W, st));
         for (int x = 0; x < E; x++) {
             const int r0 = s->h_off[x], cnt = s->h_off[x + 1] - r0;
             if (cnt > 0)
-                QIE_TRY(dense_on(b, s->abf + (int64_t)r0 * W, true, s->xg + (int64_t)r0 * W, W,
+                QIE_TRY(dense_on(b, s->xg_bf + (int64_t)r0 * W, true, s->xg + (int64_t)r0 * W, W,
                                  (const uint16_t*)L.w_gu + (int64_t)x * 2 * ff * W, s->gu + (int64_t)r0 * 2 * ff, 2 * ff, cnt,
                                  2 * ff, W));
         }
-        QIE_TRY(lay::silu_mul(s->gu, s->act, n, ff, st));
-        QIE_TRY(lay::rows_to_bf16_strided(s->act, ff, s->abf, ff, n, ff, st));
+        QIE_TRY(lay::silu_mul(s->gu, s->act, s->act_bf, n, ff, st));
         for (int x = 0; x < E; x++) {
             const int r0 = s->h_off[x], cnt = s->h_off[x + 1] - r0;
             if (cnt > 0)
-                QIE_TRY(dense_on(b, s->abf + (int64_t)r0 * ff, true, s->act + (int64_t)r0 * ff, ff,
+                QIE_TRY(dense_on(b, s->act_bf + (int64_t)r0 * ff, true, s->act + (int64_t)r0 * ff, ff,
                                  (const uint16_t*)L.w_down + (int64_t)x * W * ff, s->yd + (int64_t)r0 * W, W, cnt, W, ff));
         }
         return lay::moe_combine(s->yd, s->slot_of, T, top, W, s->ffo, st);
     }
     QIE_TRY(lin(e, s->xg, W, L.w_gu, W, s->gu, 2 * ff, n, 2 * ff, W, E, 0, (int64_t)2 * ff * W, 0, s->off));
-    QIE_TRY(lay::silu_mul(s->gu, s->act, n, ff, st));
+    QIE_TRY(lay::silu_mul(s->gu, s->act, nullptr, n, ff, st));
     QIE_TRY(lin(e, s->act, ff, L.w_down, ff, s->yd, W, n, W, ff, E, 0, (int64_t)W * ff, 0, s->off));
     return lay::moe_combine(s->yd, s->slot_of, T, top, W, s->ffo, st);
 }
 
-static int enq_layer(qie_batch* b, int i, const float* xin, int T, const float** xout) {
+static int enq_layer(qie_batch* b, int i, const float* xin, const uint16_t* xin_bf, int T, const float** xout,
+                     const uint16_t** xout_bf) {
     const qie_engine* e = b->e;
     const LayeredModel* m = e->lm;
     const LayerDev& L = m->L[i];
@@ -537,22 +543,24 @@ static int enq_layer(qie_batch* b, int i, const float* xin, int T, const float**
     hipStream_t st = e->stream;
     const int64_t plane = s->cap * W;
     float* result = s->stack + (int64_t)(i + 1) * plane;
-    QIE_TRY(enq_input_proj(b, i, xin, T));
+    QIE_TRY(enq_input_proj(b, i, xin, T, xin_bf));
     QIE_TRY(enq_latent_post(b, i, T));
     QIE_TRY(enq_absorb(b, i, T));
     QIE_TRY(enq_attention(b, i, T));
     QIE_TRY(enq_mixer_out(b, i, T));
     const bool has_ff = L.d.ff_kind != QIE_FF_NONE;
-    QIE_TRY(lay::postnorm_add(xin, s->mix, has_ff ? s->y : result, T, W, L.g1, m->a.norm_eps, st));
+    QIE_TRY(lay::postnorm_add(xin, s->mix, has_ff ? s->y : result, has_ff ? s->y_bf : nullptr, T, W, L.g1, m->a.norm_eps, st));
     if (has_ff) {
         QIE_TRY(enq_ff(b, i, T));
-        QIE_TRY(lay::postnorm_add(s->y, s->ffo, result, T, W, L.g2, m->a.norm_eps, st));
+        QIE_TRY(lay::postnorm_add(s->y, s->ffo, result, nullptr, T, W, L.g2, m->a.norm_eps, st));
     }
     if (m->a.depth_mix) {
-        QIE_TRY(lay::depth_mix(s->stack, plane, L.dwa, i + 2, s->x, (int64_t)T * W, st));
+        QIE_TRY(lay::depth_mix(s->stack, plane, L.dwa, i + 2, s->x, s->x_bf, (int64_t)T * W, st));
         *xout = s->x;
+        *xout_bf = s->x_bf;
     } else {
         *xout = result;
+        *xout_bf = nullptr;
     }
     if (s->keep_on && s->keep)
         QIE_HIP(hipMemcpyAsync(s->keep + (int64_t)i * plane, *xout, (size_t)T * W * 4, hipMemcpyDeviceToDevice, st));
@@ -564,24 +572,26 @@ static int enq_forward(qie_batch* b, int T, int n_want) {
     const LayeredModel* m = e->lm;
     LayeredBatch* s = b->lb;
     const int W = m->a.width;
-    QIE_TRY(lay::embed_rows(m->embed, m->f32, s->tok, s->stack, T, W, m->a.vocab, e->stream));
+    QIE_TRY(lay::embed_rows(m->embed, m->f32, s->tok, s->stack, s->x_bf, T, W, m->a.vocab, e->stream));
     const float* x = s->stack;
-    for (int i = 0; i < m->a.n_layers; i++) QIE_TRY(enq_layer(b, i, x, T, &x));
+    const uint16_t* x_bf = s->x_bf;
+    for (int i = 0; i < m->a.n_layers; i++) QIE_TRY(enq_layer(b, i, x, x_bf, T, &x, &x_bf));
     if (n_want > 0) {
-        QIE_TRY(lay::final_rows(x, s->want, s->xn, n_want, W, m->g_final, m->a.norm_eps, e->stream));
-        QIE_TRY(dense(b, s->xn, W, m->head, s->logits, m->a.vocab, n_want, m->a.vocab, W));
+        QIE_TRY(lay::final_rows(x, s->want, s->xn, s->xn_bf, n_want, W, m->g_final, m->a.norm_eps, e->stream));
+        QIE_TRY(dense(b, s->xn, W, m->head, s->logits, m->a.vocab, n_want, m->a.vocab, W, s->xn_bf));
     }
     return 0;
 }
 
 static void lb_free(LayeredBatch* s) {
     void* ps[] = {s->stack, s->x, s->proj, s->qabs, s->olat, s->ov, s->mix, s->y, s->gu, s->act, s->ffo, s->xg, s->yd, s->score,
-                  s->row_slot, s->row_pos, s->tok, s->sel, s->cnt, s->off, s->slot_of, s->keep, s->abf};
+                  s->row_slot, s->row_pos, s->tok, s->sel, s->cnt, s->off, s->slot_of, s->keep, s->abf,
+                  s->x_bf, s->y_bf, s->ov_bf, s->act_bf, s->xg_bf};
     for (void* p : ps)
         if (p) hipFree(p);
     s->stack = s->x = s->proj = s->qabs = s->olat = s->ov = s->mix = s->y = s->gu = s->act = s->ffo = s->xg = s->yd = s->score =
         s->keep = nullptr;
-    s->abf = nullptr;
+    s->abf = s->x_bf = s->y_bf = s->ov_bf = s->act_bf = s->xg_bf = nullptr;
     s->row_slot = s->row_pos = s->tok = s->sel = s->cnt = s->off = s->slot_of = nullptr;
     s->cap = 0;
 }
@@ -618,7 +628,14 @@ static int ensure_rows(qie_batch* b, int64_t T) {
         A((void**)&s->row_slot, cap);
         A((void**)&s->row_pos, cap);
         A((void**)&s->tok, cap);
-        if (!m->f32) A((void**)&s->abf, cap * s->m_abf + 64, 2);
+        if (!m->f32) {
+            A((void**)&s->abf, cap * s->m_abf + 64, 2);
+            A((void**)&s->x_bf, cap * W, 2);
+            A((void**)&s->y_bf, cap * W, 2);
+            A((void**)&s->ov_bf, cap * s->m_hv, 2);
+            A((void**)&s->act_bf, cap * std::max<int64_t>(s->m_act, 1), 2);
+            A((void**)&s->xg_bf, cap * std::max<int64_t>(s->m_top, 1) * W, 2);
+        }
         if (s->keep_on) A((void**)&s->keep, L * cap * W);
         if (rc) return rc;
         s->cap = cap;
@@ -639,14 +656,16 @@ static int ensure_want(qie_batch* b, int64_t n) {
     const LayeredModel* m = b->e->lm;
     if (n <= s->want_cap) return 0;
     QIE_HIP(hipStreamSynchronize(b->e->stream));
-    void* ps[] = {s->want, s->xn, s->logits, s->logits_bf, s->d_ids, s->d_step};
+    void* ps[] = {s->want, s->xn, s->logits, s->logits_bf, s->d_ids, s->d_step, s->xn_bf};
     for (void* p : ps)
         if (p) hipFree(p);
+    s->xn_bf = nullptr;
     s->want = nullptr; s->xn = nullptr; s->logits = nullptr; s->logits_bf = nullptr; s->d_ids = nullptr; s->d_step = nullptr;
     s->want_cap = 0;
     const int64_t cap = (n + 15) / 16 * 16, V = m->a.vocab;
     QIE_TRY(dmalloc((void**)&s->want, cap * 4));
     QIE_TRY(dmalloc((void**)&s->xn, cap * m->a.width * 4));
+    if (!m->f32) QIE_TRY(dmalloc((void**)&s->xn_bf, cap * m->a.width * 2));
     QIE_TRY(dmalloc((void**)&s->logits, cap * V * 4));
     QIE_TRY(dmalloc((void**)&s->logits_bf, cap * V * 2));
     QIE_TRY(dmalloc((void**)&s->d_ids, cap * 4));
@@ -734,7 +753,7 @@ void layered_batch_destroy(qie_batch* b) {
     LayeredBatch* s = b->lb;
     if (!s) return;
     lb_free(s);
-    void* ps[] = {s->want, s->xn, s->logits, s->logits_bf, s->d_ids, s->d_step, s->d_groups, s->part_o, s->part_ml};
+    void* ps[] = {s->want, s->xn, s->logits, s->logits_bf, s->d_ids, s->d_step, s->d_groups, s->part_o, s->part_ml, s->xn_bf};
     for (void* p : ps)
         if (p) hipFree(p);
     if (s->h_stage) hipHostFree(s->h_stage);
@@ -967,7 +986,7 @@ int qie_batch_time_stage(qie_batch* b, int32_t which, int32_t layer, int32_t ite
             case 0: return enq_forward(b, T, s->last_want);
             case 1: return enq_attention(b, layer, T);
             case 2:
-                QIE_TRY(enq_input_proj(b, layer, xin, T));
+                QIE_TRY(enq_input_proj(b, layer, xin, T, s->x_bf));
                 QIE_TRY(enq_absorb(b, layer, T));
                 return enq_mixer_out(b, layer, T);
             default: return enq_ff(b, layer, T);

@@ -272,17 +272,23 @@ int linear(const LinearP& p, bool w_f32, hipStream_t st) {
 
 // ------------------------------------------------------------------ embedding rows
 template <typename TW>
-__global__ __launch_bounds__(256) void embed_rows_kernel(const TW* E, const int32_t* tok, float* out, int W, int vocab) {
+__global__ __launch_bounds__(256) void embed_rows_kernel(const TW* E, const int32_t* tok, float* out, uint16_t* out_bf, int W,
+                                                         int vocab) {
     const int t = blockIdx.x;
     int id = tok[t];
     if (id < 0 || id >= vocab) id = 0;
-    for (int w = threadIdx.x; w < W; w += 256) out[(int64_t)t * W + w] = ldf<TW>(E, (int64_t)id * W + w);
+    for (int w = threadIdx.x; w < W; w += 256) {
+        const float v = ldf<TW>(E, (int64_t)id * W + w);
+        out[(int64_t)t * W + w] = v;
+        if (out_bf) out_bf[(int64_t)t * W + w] = f2bf(v);
+    }
 }
-int embed_rows(const void* E, bool w_f32, const int32_t* tok, float* out, int T, int W, int vocab, hipStream_t st) {
+int embed_rows(const void* E, bool w_f32, const int32_t* tok, float* out, uint16_t* out_bf, int T, int W, int vocab,
+               hipStream_t st) {
     if (w_f32)
-        hipLaunchKernelGGL(embed_rows_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)E, tok, out, W, vocab);
+        hipLaunchKernelGGL(embed_rows_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)E, tok, out, out_bf, W, vocab);
     else
-        hipLaunchKernelGGL(embed_rows_kernel<uint16_t>, dim3(T), dim3(256), 0, st, (const uint16_t*)E, tok, out, W, vocab);
+        hipLaunchKernelGGL(embed_rows_kernel<uint16_t>, dim3(T), dim3(256), 0, st, (const uint16_t*)E, tok, out, out_bf, W, vocab);
     QIE_LAUNCH_CHECK();
     return 0;
 }
@@ -442,25 +448,27 @@ int latent_attention(const LatentAttnP& p, bool cache_f32, int T, hipStream_t st
 
 // ------------------------------------------------------------------ per-head output gate
 // v[t, h, :] *= sigmoid(gate[t, h]); gate logits sit in the projection row at column g_col
-__global__ __launch_bounds__(256) void head_gate_kernel(float* v, const float* proj, int64_t ld, int g_col, int heads, int vd,
-                                                        int64_t n) {
+__global__ __launch_bounds__(256) void head_gate_kernel(float* v, uint16_t* v_bf, const float* proj, int64_t ld, int g_col, int heads,
+                                                        int vd, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
     const int64_t t = i / ((int64_t)heads * vd);
     const int h = (int)((i / vd) % heads);
     const float g = proj[t * ld + g_col + h];
-    v[i] *= 1.0f / (1.0f + expf(-g));
+    const float o = v[i] * (1.0f / (1.0f + expf(-g)));
+    v[i] = o;
+    if (v_bf) v_bf[i] = f2bf(o);
 }
-int head_gate(float* v, const float* proj, int64_t ld, int g_col, int heads, int vd, int T, hipStream_t st) {
+int head_gate(float* v, uint16_t* v_bf, const float* proj, int64_t ld, int g_col, int heads, int vd, int T, hipStream_t st) {
     const int64_t n = (int64_t)T * heads * vd;
-    hipLaunchKernelGGL(head_gate_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, v, proj, ld, g_col, heads, vd, n);
+    hipLaunchKernelGGL(head_gate_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, v, v_bf, proj, ld, g_col, heads, vd, n);
     QIE_LAUNCH_CHECK();
     return 0;
 }
 
 // ------------------------------------------------------------------ norm on the sublayer output
-__global__ __launch_bounds__(256) void postnorm_add_kernel(const float* x, const float* v, float* y, int W, float gain,
-                                                           float eps) {
+__global__ __launch_bounds__(256) void postnorm_add_kernel(const float* x, const float* v, float* y, uint16_t* y_bf, int W,
+                                                           float gain, float eps) {
     __shared__ float red[4];
     const int64_t t = blockIdx.x;
     float ss = 0.f;
@@ -470,17 +478,21 @@ __global__ __launch_bounds__(256) void postnorm_add_kernel(const float* x, const
     }
     ss = block_sum256(ss, red);
     const float inv = gain / sqrtf(ss / (float)W + eps);
-    for (int i = threadIdx.x; i < W; i += 256) y[t * W + i] = (x ? x[t * W + i] : 0.f) + v[t * W + i] * inv;
+    for (int i = threadIdx.x; i < W; i += 256) {
+        const float o = (x ? x[t * W + i] : 0.f) + v[t * W + i] * inv;
+        y[t * W + i] = o;
+        if (y_bf) y_bf[t * W + i] = f2bf(o);
+    }
 }
-int postnorm_add(const float* x, const float* v, float* y, int T, int W, float gain, float eps, hipStream_t st) {
-    hipLaunchKernelGGL(postnorm_add_kernel, dim3(T), dim3(256), 0, st, x, v, y, W, gain, eps);
+int postnorm_add(const float* x, const float* v, float* y, uint16_t* y_bf, int T, int W, float gain, float eps, hipStream_t st) {
+    hipLaunchKernelGGL(postnorm_add_kernel, dim3(T), dim3(256), 0, st, x, v, y, y_bf, W, gain, eps);
     QIE_LAUNCH_CHECK();
     return 0;
 }
 
 // rows picked by index, normed with one gain: out[i] = gain * x[rows[i]] / rms
-__global__ __launch_bounds__(256) void final_rows_kernel(const float* x, const int32_t* rows, float* out, int W, float gain,
-                                                         float eps) {
+__global__ __launch_bounds__(256) void final_rows_kernel(const float* x, const int32_t* rows, float* out, uint16_t* out_bf, int W,
+                                                         float gain, float eps) {
     __shared__ float red[4];
     const int64_t t = rows[blockIdx.x];
     float ss = 0.f;
@@ -490,10 +502,15 @@ __global__ __launch_bounds__(256) void final_rows_kernel(const float* x, const i
     }
     ss = block_sum256(ss, red);
     const float inv = gain / sqrtf(ss / (float)W + eps);
-    for (int i = threadIdx.x; i < W; i += 256) out[(int64_t)blockIdx.x * W + i] = x[t * W + i] * inv;
+    for (int i = threadIdx.x; i < W; i += 256) {
+        const float o = x[t * W + i] * inv;
+        out[(int64_t)blockIdx.x * W + i] = o;
+        if (out_bf) out_bf[(int64_t)blockIdx.x * W + i] = f2bf(o);
+    }
 }
-int final_rows(const float* x, const int32_t* rows, float* out, int n, int W, float gain, float eps, hipStream_t st) {
-    hipLaunchKernelGGL(final_rows_kernel, dim3(n), dim3(256), 0, st, x, rows, out, W, gain, eps);
+int final_rows(const float* x, const int32_t* rows, float* out, uint16_t* out_bf, int n, int W, float gain, float eps,
+               hipStream_t st) {
+    hipLaunchKernelGGL(final_rows_kernel, dim3(n), dim3(256), 0, st, x, rows, out, out_bf, W, gain, eps);
     QIE_LAUNCH_CHECK();
     return 0;
 }
@@ -501,33 +518,37 @@ int final_rows(const float* x, const int32_t* rows, float* out, int n, int W, fl
 // ------------------------------------------------------------------ depth-weighted average
 // x[t, w] = sum_{j < n} a[j] X[j][t, w]; X[j] at stack + j * stride
 __global__ __launch_bounds__(256) void depth_mix_kernel(const float* stack, int64_t stride, const float* a, int n, float* x,
-                                                        int64_t count) {
+                                                        uint16_t* x_bf, int64_t count) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= count) return;
     float s = 0.f;
     for (int j = 0; j < n; j++) s = fmaf(a[j], stack[j * stride + i], s);
     x[i] = s;
+    if (x_bf) x_bf[i] = f2bf(s);
 }
-int depth_mix(const float* stack, int64_t stride, const float* a, int n, float* x, int64_t count, hipStream_t st) {
-    hipLaunchKernelGGL(depth_mix_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st, stack, stride, a, n, x, count);
+int depth_mix(const float* stack, int64_t stride, const float* a, int n, float* x, uint16_t* x_bf, int64_t count, hipStream_t st) {
+    hipLaunchKernelGGL(depth_mix_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st, stack, stride, a, n, x, x_bf,
+                       count);
     QIE_LAUNCH_CHECK();
     return 0;
 }
 
 // ------------------------------------------------------------------ gated activation
 // a[m, j] = silu(gu[m, j]) * gu[m, ff + j]
-__global__ __launch_bounds__(256) void silu_mul_kernel(const float* gu, float* a, int ff, int64_t n) {
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float* gu, float* a, uint16_t* a_bf, int ff, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
     const int64_t m = i / ff;
     const int j = (int)(i % ff);
     const float g = gu[m * 2 * ff + j], u = gu[m * 2 * ff + ff + j];
-    a[i] = g / (1.0f + expf(-g)) * u;
+    const float o = g / (1.0f + expf(-g)) * u;
+    a[i] = o;
+    if (a_bf) a_bf[i] = f2bf(o);
 }
-int silu_mul(const float* gu, float* a, int64_t M, int ff, hipStream_t st) {
+int silu_mul(const float* gu, float* a, uint16_t* a_bf, int64_t M, int ff, hipStream_t st) {
     const int64_t n = M * ff;
     if (n == 0) return 0;
-    hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, gu, a, ff, n);
+    hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, gu, a, a_bf, ff, n);
     QIE_LAUNCH_CHECK();
     return 0;
 }
@@ -624,14 +645,19 @@ int moe_group(const int32_t* sel, int n, int E, int32_t* cnt, int32_t* off, int3
 }
 // xg[slot_of[i], :] = score[i] * y[i / top, :]
 __global__ __launch_bounds__(256) void moe_gather_kernel(const float* y, const float* score, const int32_t* slot_of, int top, int W,
-                                                         float* xg) {
+                                                         float* xg, uint16_t* xg_bf) {
     const int64_t i = blockIdx.x;
     const int64_t t = i / top, d = slot_of[i];
     const float s = score[i];
-    for (int w = threadIdx.x; w < W; w += 256) xg[d * W + w] = s * y[t * W + w];
+    for (int w = threadIdx.x; w < W; w += 256) {
+        const float o = s * y[t * W + w];
+        xg[d * W + w] = o;
+        if (xg_bf) xg_bf[d * W + w] = f2bf(o);
+    }
 }
-int moe_gather(const float* y, const float* score, const int32_t* slot_of, int T, int top, int W, float* xg, hipStream_t st) {
-    hipLaunchKernelGGL(moe_gather_kernel, dim3(T * top), dim3(256), 0, st, y, score, slot_of, top, W, xg);
+int moe_gather(const float* y, const float* score, const int32_t* slot_of, int T, int top, int W, float* xg, uint16_t* xg_bf,
+               hipStream_t st) {
+    hipLaunchKernelGGL(moe_gather_kernel, dim3(T * top), dim3(256), 0, st, y, score, slot_of, top, W, xg, xg_bf);
     QIE_LAUNCH_CHECK();
     return 0;
 }

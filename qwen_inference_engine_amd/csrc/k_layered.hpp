@@ -96,17 +96,22 @@ constexpr int kLatentQG = 1;   // 2 measured slower at kv_rank 256 (one wave per
 bool latent_attention_mfma_fits(int R, int rot);
 int latent_attention_mfma(const LatentAttnMfmaP& p, hipStream_t st);
 
-int embed_rows(const void* E, bool w_f32, const int32_t* tok, float* out, int T, int W, int vocab, hipStream_t st);
-int head_gate(float* v, const float* proj, int64_t ld, int g_col, int heads, int vd, int T, hipStream_t st);
+// The producers below also write the bf16 image of their result when the *_bf pointer is set
+// (bf16 engines: the next product reads it; no separate rounding pass).
+int embed_rows(const void* E, bool w_f32, const int32_t* tok, float* out, uint16_t* out_bf, int T, int W, int vocab,
+               hipStream_t st);
+int head_gate(float* v, uint16_t* v_bf, const float* proj, int64_t ld, int g_col, int heads, int vd, int T, hipStream_t st);
 // y = (x ? x : 0) + gain * v / sqrt(mean(v^2) + eps), rows of W
-int postnorm_add(const float* x, const float* v, float* y, int T, int W, float gain, float eps, hipStream_t st);
-int final_rows(const float* x, const int32_t* rows, float* out, int n, int W, float gain, float eps, hipStream_t st);
-int depth_mix(const float* stack, int64_t stride, const float* a, int n, float* x, int64_t count, hipStream_t st);
-int silu_mul(const float* gu, float* a, int64_t M, int ff, hipStream_t st);
+int postnorm_add(const float* x, const float* v, float* y, uint16_t* y_bf, int T, int W, float gain, float eps, hipStream_t st);
+int final_rows(const float* x, const int32_t* rows, float* out, uint16_t* out_bf, int n, int W, float gain, float eps,
+               hipStream_t st);
+int depth_mix(const float* stack, int64_t stride, const float* a, int n, float* x, uint16_t* x_bf, int64_t count, hipStream_t st);
+int silu_mul(const float* gu, float* a, uint16_t* a_bf, int64_t M, int ff, hipStream_t st);
 int route_sigmoid_topk(const float* y, const void* Wr, bool w_f32, int T, int W, int E, int top, int32_t* sel, float* score,
                        hipStream_t st);
 int moe_group(const int32_t* sel, int n, int E, int32_t* cnt, int32_t* off, int32_t* slot_of, hipStream_t st);
-int moe_gather(const float* y, const float* score, const int32_t* slot_of, int T, int top, int W, float* xg, hipStream_t st);
+int moe_gather(const float* y, const float* score, const int32_t* slot_of, int T, int top, int W, float* xg, uint16_t* xg_bf,
+               hipStream_t st);
 int moe_combine(const float* yd, const int32_t* slot_of, int T, int top, int W, float* f, hipStream_t st);
 int argmax_rows(const float* x, int M, int64_t V, int32_t* ids, hipStream_t st);
 int rows_to_bf16(const float* x, uint16_t* y, int64_t n, hipStream_t st);
