@@ -92,6 +92,11 @@ struct LayeredBatch {
     float *part_o = nullptr, *part_ml = nullptr;
     int64_t part_cap = 0;         // (group, split) units the partials hold
     bool interleaved = false;     // the cache pages carry the key-interleaved copy of c
+    // per-expert products of prompt-sized steps run on side streams beside the engine's (every
+    // expert's GEMM alone covers a fraction of the chip); default priority, joined by events
+    static constexpr int kSide = 3;
+    hipStream_t side[kSide] = {nullptr, nullptr, nullptr};
+    hipEvent_t ev_fork = nullptr, ev_join[kSide] = {nullptr, nullptr, nullptr};
     std::vector<int32_t> h_off;   // host copy of the expert row offsets (prompt-sized steps)
     int32_t *row_slot = nullptr, *row_pos = nullptr, *tok = nullptr, *want = nullptr, *sel = nullptr, *cnt = nullptr,
             *off = nullptr, *slot_of = nullptr, *d_ids = nullptr, *d_step = nullptr;
@@ -311,20 +316,22 @@ static bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 // the model runs bf16 operands and the shapes fit them (K a multiple of 8, 16-byte aligned
 // operands); `abf` receives the bf16 image of A, row stride K.  Else the plain kernel.
 static int dense_on(qie_batch* b, uint16_t* abf, bool staged, const float* A, int64_t lda, const void* Wt, float* Y, int64_t ldy,
-                    int M, int N, int K) {
+                    int M, int N, int K, hipStream_t on = nullptr) {
     const qie_engine* e = b->e;
+    const hipStream_t st = on ? on : e->stream;
     if (!e->lm->f32 && abf && K % 8 == 0 && al16(Wt) && al16(abf)) {
-        if (!staged) QIE_TRY(lay::rows_to_bf16_strided(A, lda, abf, K, M, K, e->stream));
+        if (!staged) QIE_TRY(lay::rows_to_bf16_strided(A, lda, abf, K, M, K, st));
         qie_linear_args a{};
         a.x = abf; a.ldx = K;
         a.w[0] = Wt; a.seg_rows[0] = N;
         a.M = M; a.K = K; a.N = N;
         a.y = Y; a.ldy = ldy;
         a.epilogue = QIE_EPI_F32;
-        const int rc = qie_linear(&a, e->stream);
+        const int rc = qie_linear(&a, st);
         if (rc != -22) return rc;   // a shape those kernels do not take: the plain kernel below
     }
-    return lin(e, A, lda, Wt, K, Y, ldy, M, N, K);
+    lay::LinearP p{A, lda, Wt, K, Y, ldy, M, N, K, 1, 0, 0, 0, e->lm->f32 ? 0 : 1, nullptr, e->lm->f32 ? 0 : 1};
+    return lay::linear(p, e->lm->f32, st);
 }
 // pre: the bf16 image of A (row stride K) when its producer wrote one
 static int dense(qie_batch* b, const float* A, int64_t lda, const void* Wt, float* Y, int64_t ldy, int M, int N, int K,
@@ -511,20 +518,40 @@ static int enq_ff(qie_batch* b, int i, int T) {
         s->h_off.resize(E + 1);
         QIE_HIP(hipMemcpyAsync(s->h_off.data(), s->off, (size_t)(E + 1) * 4, hipMemcpyDeviceToHost, st));
         QIE_HIP(hipStreamSynchronize(st));
+        // experts round-robin over the engine's stream and the side streams, forked and joined
+        // by events around each of the two product phases
+        auto fork = [&]() -> int {
+            QIE_HIP(hipEventRecord(s->ev_fork, st));
+            for (int i = 0; i < LayeredBatch::kSide; i++) QIE_HIP(hipStreamWaitEvent(s->side[i], s->ev_fork, 0));
+            return 0;
+        };
+        auto join = [&]() -> int {
+            for (int i = 0; i < LayeredBatch::kSide; i++) {
+                QIE_HIP(hipEventRecord(s->ev_join[i], s->side[i]));
+                QIE_HIP(hipStreamWaitEvent(st, s->ev_join[i], 0));
+            }
+            return 0;
+        };
+        auto lane_of = [&](int x) { return x % (LayeredBatch::kSide + 1) == 0 ? st : s->side[x % (LayeredBatch::kSide + 1) - 1]; };
+        QIE_TRY(fork());
         for (int x = 0; x < E; x++) {
             const int r0 = s->h_off[x], cnt = s->h_off[x + 1] - r0;
             if (cnt > 0)
                 QIE_TRY(dense_on(b, s->xg_bf + (int64_t)r0 * W, true, s->xg + (int64_t)r0 * W, W,
                                  (const uint16_t*)L.w_gu + (int64_t)x * 2 * ff * W, s->gu + (int64_t)r0 * 2 * ff, 2 * ff, cnt,
-                                 2 * ff, W));
+                                 2 * ff, W, lane_of(x)));
         }
+        QIE_TRY(join());
         QIE_TRY(lay::silu_mul(s->gu, s->act, s->act_bf, n, ff, st));
+        QIE_TRY(fork());
         for (int x = 0; x < E; x++) {
             const int r0 = s->h_off[x], cnt = s->h_off[x + 1] - r0;
             if (cnt > 0)
                 QIE_TRY(dense_on(b, s->act_bf + (int64_t)r0 * ff, true, s->act + (int64_t)r0 * ff, ff,
-                                 (const uint16_t*)L.w_down + (int64_t)x * W * ff, s->yd + (int64_t)r0 * W, W, cnt, W, ff));
+                                 (const uint16_t*)L.w_down + (int64_t)x * W * ff, s->yd + (int64_t)r0 * W, W, cnt, W, ff,
+                                 lane_of(x)));
         }
+        QIE_TRY(join());
         return lay::moe_combine(s->yd, s->slot_of, T, top, W, s->ffo, st);
     }
     QIE_TRY(lin(e, s->xg, W, L.w_gu, W, s->gu, 2 * ff, n, 2 * ff, W, E, 0, (int64_t)2 * ff * W, 0, s->off));
@@ -741,6 +768,14 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
         if (he != hipSuccess) rc = fail((int)he, "batch init: %s", hipGetErrorString(he));
     }
     if (!rc) rc = flush_table(b);
+    if (!rc) {
+        hipError_t he = hipEventCreateWithFlags(&s->ev_fork, hipEventDisableTiming);
+        for (int i = 0; i < LayeredBatch::kSide && he == hipSuccess; i++) {
+            he = hipStreamCreateWithFlags(&s->side[i], hipStreamNonBlocking);
+            if (he == hipSuccess) he = hipEventCreateWithFlags(&s->ev_join[i], hipEventDisableTiming);
+        }
+        if (he != hipSuccess) rc = fail((int)he, "batch init (side streams): %s", hipGetErrorString(he));
+    }
     if (rc) {
         qie_batch_destroy(b);
         return rc;
@@ -757,6 +792,12 @@ void layered_batch_destroy(qie_batch* b) {
     for (void* p : ps)
         if (p) hipFree(p);
     if (s->h_stage) hipHostFree(s->h_stage);
+    for (int i = 0; i < LayeredBatch::kSide; i++) {
+        if (s->side[i]) hipStreamSynchronize(s->side[i]);
+        if (s->ev_join[i]) hipEventDestroy(s->ev_join[i]);
+        if (s->side[i]) hipStreamDestroy(s->side[i]);
+    }
+    if (s->ev_fork) hipEventDestroy(s->ev_fork);
     delete s;
     b->lb = nullptr;
 }

@@ -112,13 +112,12 @@ def test_ragged_planner_budget_order_and_completion():
     # steps 1-2 read 20 tokens of r0; step 3 ends both prompts; r2 takes r1's slot once r1 is done
     assert out == {r0: [1003, 1004, 1005], r1: [1003, 1004], r2: [1005, 1006]}
     steps = eng.b.steps
-    # step 1: both prompts are new; the budget of 10 rows goes to slot 0 first, then slot 1
+    # step 1: both prompts are new; the budget of 10 rows goes to slot 0 first, nothing is left for slot 1
     assert steps[0] == ([(0, list(range(100, 110)))], [])
-    # step 2: slot 0 continues, slot 1 gets nothing (budget) ... every step stays within 10 rows
+    # every step stays within 10 rows, entries in slot order
     for entries, want in steps:
         assert sum(len(t) for _, t in entries) <= 10
         assert [s for s, _ in entries] == sorted(s for s, _ in entries)
-    # a decoding request is never starved by prompts: once r1 decodes it is in every step until done
     fed = {0: [], 1: []}
     for entries, _ in steps:
         for s, t in entries:
