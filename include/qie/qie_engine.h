@@ -261,8 +261,8 @@ int qie_batch_debug_step(qie_batch* b, const qie_sampling* smp, int32_t* next_id
  * W_uv applied to the softmax-weighted sum of c), for prompts and decoding alike.
  * Feed-forward: none, dense gated SiLU, or a mixture of `experts` gated-SiLU experts with a
  * sigmoid router (fp32) whose `top` largest scores, not renormalised, scale the experts' input.
- * Layer: y = x + g1 * rms(mixer(x)); z = y + g2 * rms(ff(y)) (scalar gains, norm on the
- * sublayer's output); the next layer's input is the depth-weighted sum over the embedding
+ * Layer: y = x + g1 * rms(mixer(x)); z = y + g2 * rms(ff(y)) (scalar gains; each branch is
+ * normed after it is computed, its input is the raw stream); the next layer's input is the depth-weighted sum over the embedding
  * output and every layer result so far. */
 enum { QIE_MIXER_LATENT_ATTENTION = 1 };
 enum { QIE_FF_NONE = 0, QIE_FF_DENSE = 1, QIE_FF_MOE = 2 };
@@ -270,7 +270,7 @@ enum { QIE_FF_NONE = 0, QIE_FF_DENSE = 1, QIE_FF_MOE = 2 };
 typedef struct qie_layer_desc {
     int32_t mixer;            /* QIE_MIXER_*                                          */
     int32_t heads, dim, rot_dim, vdim, kv_rank;
-    int32_t window;           /* position i sees j with 0 <= i - j < window           */
+    int32_t window;           /* query at position i attends keys i - window < j <= i */
     int32_t kv_from;          /* -1: own W_dkv; else the layer whose cache rows it reads */
     int32_t rot_dims;         /* rotated coordinates of a rotated part (even, <= rot_dim) */
     float rot_base, scale;
@@ -311,6 +311,11 @@ int qie_batch_step(qie_batch* b, int32_t n_entries, const int32_t* slots, const 
  * (top_k <= 1 or temperature <= 0): arg-max of the fp32 row, ties to the lowest id; otherwise
  * qie_sample on the rows rounded to bf16, as the sampler reads them. */
 int qie_batch_step_sample(qie_batch* b, const qie_sampling* s, int32_t* host_ids);
+/* Steps of at most 16 rows replay a hipGraph of their shape (rows, wanted rows, row groups),
+ * captured the second time the shape is seen, when the engine was created with use_graph; every
+ * per-step value (ids, slots, positions, block table, row groups) is read from device memory.
+ * Instantiated graphs and replays so far: */
+int qie_batch_step_graphs(qie_batch* b, int32_t* n_graphs, int64_t* n_replays);
 /* Diagnostics: enable != 0 makes every following step keep the stream after each layer;
  * qie_batch_step_layers copies the last step's [n_layers][rows][width] fp32 to host_out. */
 int qie_batch_keep_layers(qie_batch* b, int32_t enable);

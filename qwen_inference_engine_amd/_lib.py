@@ -218,6 +218,7 @@ SIGNATURES = [
     ("qie_engine_finalize_weights", C.c_int, [_P]),
     ("qie_batch_step", C.c_int, [_P, _I32, _PI32, _PI32, _PI32, _I32, _PI32, _PF]),
     ("qie_batch_step_sample", C.c_int, [_P, C.POINTER(SamplingC), _PI32]),
+    ("qie_batch_step_graphs", C.c_int, [_P, _PI32, _PI64]),
     ("qie_batch_keep_layers", C.c_int, [_P, _I32]),
     ("qie_batch_step_layers", C.c_int, [_P, _PF, _I64]),
     ("qie_batch_time_stage", C.c_int, [_P, _I32, _I32, _I32, _PD]),

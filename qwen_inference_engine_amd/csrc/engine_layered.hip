@@ -97,6 +97,11 @@ struct LayeredBatch {
     static constexpr int kSide = 3;
     hipStream_t side[kSide] = {nullptr, nullptr, nullptr};
     hipEvent_t ev_fork = nullptr, ev_join[kSide] = {nullptr, nullptr, nullptr};
+    // hipGraphs of small steps (decoding): one per step shape (rows, wanted rows, row groups per head
+    // count), captured the second time a shape is seen (the first run makes every allocation);
+    // every per-step value is read from device memory, so a replay only needs the uploads before it
+    std::map<std::vector<int>, std::pair<int, hipGraphExec_t>> graphs;   // shape -> (times seen, exec or null)
+    int64_t graph_replays = 0;
     std::vector<int32_t> h_off;   // host copy of the expert row offsets (prompt-sized steps)
     int32_t *row_slot = nullptr, *row_pos = nullptr, *tok = nullptr, *want = nullptr, *sel = nullptr, *cnt = nullptr,
             *off = nullptr, *slot_of = nullptr, *d_ids = nullptr, *d_step = nullptr;
@@ -305,6 +310,8 @@ static int lin(const qie_engine* e, const float* A, int64_t lda, const void* Wt,
     return lay::linear(p, e->lm->f32, e->stream);
 }
 
+static void drop_graphs(LayeredBatch* s);
+
 // Row count from which a step's expert products run per expert on the MFMA kernels (one
 // device-to-host copy of the expert offsets per routed layer); below it the grouped kernel runs
 // without a host round trip.
@@ -412,7 +419,11 @@ static int enq_attention(qie_batch* b, int i, int T) {
         const int nb = d.window / 32 + 2;
         S = std::max(1, std::min({S, nb, 64}));
         if ((int64_t)ng * S > s->part_cap) {
+            hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+            QIE_REQUIRE(hipStreamIsCapturing(e->stream, &cs) == hipSuccess && cs == hipStreamCaptureStatusNone,
+                        "latent attention: scratch growth inside a capture");
             QIE_HIP(hipStreamSynchronize(e->stream));
+            drop_graphs(s);
             if (s->part_o) hipFree(s->part_o);
             if (s->part_ml) hipFree(s->part_ml);
             s->part_o = s->part_ml = nullptr;
@@ -467,6 +478,7 @@ static int build_groups(qie_batch* b, int n_entries, const int32_t* counts) {
     }
     if ((int64_t)s->h_groups.size() > s->groups_cap) {
         QIE_HIP(hipStreamSynchronize(b->e->stream));
+        drop_graphs(s);
         if (s->d_groups) hipFree(s->d_groups);
         s->d_groups = nullptr;
         s->groups_cap = 0;
@@ -610,7 +622,14 @@ static int enq_forward(qie_batch* b, int T, int n_want) {
     return 0;
 }
 
+static void drop_graphs(LayeredBatch* s) {
+    for (auto& g : s->graphs)
+        if (g.second.second) hipGraphExecDestroy(g.second.second);
+    s->graphs.clear();
+}
+
 static void lb_free(LayeredBatch* s) {
+    drop_graphs(s);   // captured launches hold these buffers' addresses
     void* ps[] = {s->stack, s->x, s->proj, s->qabs, s->olat, s->ov, s->mix, s->y, s->gu, s->act, s->ffo, s->xg, s->yd, s->score,
                   s->row_slot, s->row_pos, s->tok, s->sel, s->cnt, s->off, s->slot_of, s->keep, s->abf,
                   s->x_bf, s->y_bf, s->ov_bf, s->act_bf, s->xg_bf};
@@ -621,6 +640,54 @@ static void lb_free(LayeredBatch* s) {
     s->abf = s->x_bf = s->y_bf = s->ov_bf = s->act_bf = s->xg_bf = nullptr;
     s->row_slot = s->row_pos = s->tok = s->sel = s->cnt = s->off = s->slot_of = nullptr;
     s->cap = 0;
+}
+
+
+// Small steps replay a captured graph of their shape; other steps, and the first run of a shape,
+// enqueue eagerly.
+static int run_forward(qie_batch* b, int T, int n_want) {
+    qie_engine* e = b->e;
+    LayeredBatch* s = b->lb;
+    const LayeredModel* m = e->lm;
+    bool can = e->opts.use_graph && T <= 16 && !s->keep_on;
+    for (const LayerDev& L : m->L)
+        if (L.d.ff_kind == QIE_FF_MOE && (int64_t)T * L.d.top >= kMoeSyncRows) can = false;   // host round trip inside
+    if (!can) return enq_forward(b, T, n_want);
+    std::vector<int> key{T, n_want};
+    for (const auto& g : s->groups) {
+        key.push_back(g.first);
+        key.push_back(g.second.first);
+        key.push_back((int)g.second.second);
+    }
+    auto& slot = s->graphs[key];
+    slot.first++;
+    if (slot.first == 1) return enq_forward(b, T, n_want);   // allocations and lazy attributes happen here
+    if (!slot.second && slot.first == 2) {
+        hipGraph_t graph = nullptr;
+        QIE_HIP(hipStreamBeginCapture(e->stream, hipStreamCaptureModeThreadLocal));
+        const int rc = enq_forward(b, T, n_want);
+        const hipError_t he = hipStreamEndCapture(e->stream, &graph);
+        if (rc || he != hipSuccess || !graph) {
+            if (graph) hipGraphDestroy(graph);
+            (void)hipGetLastError();
+            if (rc) return rc;
+            return enq_forward(b, T, n_want);   // this shape stays eager
+        }
+        hipGraphExec_t ex = nullptr;
+        const hipError_t hi = hipGraphInstantiate(&ex, graph, nullptr, nullptr, 0);
+        hipGraphDestroy(graph);
+        if (hi != hipSuccess || !ex) {
+            (void)hipGetLastError();
+            return enq_forward(b, T, n_want);
+        }
+        slot.second = ex;
+    }
+    if (slot.second) {
+        QIE_HIP(hipGraphLaunch(slot.second, e->stream));
+        s->graph_replays++;
+        return 0;
+    }
+    return enq_forward(b, T, n_want);
 }
 
 static int ensure_rows(qie_batch* b, int64_t T) {
@@ -667,6 +734,7 @@ static int ensure_rows(qie_batch* b, int64_t T) {
         if (rc) return rc;
         s->cap = cap;
     }
+    if (s->keep_on && !s->keep) drop_graphs(s);
     if (s->keep_on && !s->keep) QIE_TRY(dmalloc((void**)&s->keep, (size_t)m->a.n_layers * s->cap * m->a.width * 4));
     if (T > s->h_stage_rows) {
         if (s->h_stage) hipHostFree(s->h_stage);
@@ -683,6 +751,7 @@ static int ensure_want(qie_batch* b, int64_t n) {
     const LayeredModel* m = b->e->lm;
     if (n <= s->want_cap) return 0;
     QIE_HIP(hipStreamSynchronize(b->e->stream));
+    drop_graphs(s);
     void* ps[] = {s->want, s->xn, s->logits, s->logits_bf, s->d_ids, s->d_step, s->xn_bf};
     for (void* p : ps)
         if (p) hipFree(p);
@@ -838,7 +907,6 @@ int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* 
     qie_engine* e = new qie_engine();
     if (opts) e->opts = *opts;
     if (e->opts.max_ctx <= 0) e->opts.max_ctx = 4096;
-    e->opts.use_graph = 0;
     e->opts.tp_size = 1;
     e->opts.tp_rank = 0;
     e->sh.tp = 1;
@@ -956,7 +1024,7 @@ int qie_batch_step(qie_batch* b, int32_t n_entries, const int32_t* slots, const 
     QIE_HIP(hipMemcpyAsync(s->tok, hs + 2 * R, (size_t)T * 4, hipMemcpyHostToDevice, st));
     QIE_TRY(build_groups(b, n_entries, counts));
     if (n_want > 0) QIE_HIP(hipMemcpyAsync(s->want, want_rows, (size_t)n_want * 4, hipMemcpyHostToDevice, st));
-    QIE_TRY(enq_forward(b, (int)T, n_want));
+    QIE_TRY(run_forward(b, (int)T, n_want));
     s->last_T = (int)T;
     s->last_want = n_want;
     s->steps++;
@@ -987,6 +1055,15 @@ int qie_batch_step_sample(qie_batch* b, const qie_sampling* smp, int32_t* host_i
     }
     QIE_HIP(hipMemcpyAsync(host_ids, s->d_ids, (size_t)n * 4, hipMemcpyDeviceToHost, st));
     QIE_HIP(hipStreamSynchronize(st));
+    return 0;
+}
+
+int qie_batch_step_graphs(qie_batch* b, int32_t* n_graphs, int64_t* n_replays) {
+    QIE_REQUIRE(b && b->lb, "qie_batch_step_graphs: a batch of a layered engine");
+    int n = 0;
+    for (const auto& g : b->lb->graphs) n += g.second.second != nullptr;
+    if (n_graphs) *n_graphs = n;
+    if (n_replays) *n_replays = b->lb->graph_replays;
     return 0;
 }
 

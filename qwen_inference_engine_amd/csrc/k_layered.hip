@@ -9,7 +9,7 @@
 //   lay::latent_attention  sliding-window attention over the latent cache in absorbed form
 //                          (scores against [c ; k_rot], output in latent space), online softmax
 //   lay::head_gate         per-head sigmoid output gate
-//   lay::postnorm_add      y = x + g * v / sqrt(mean(v^2) + eps): norm on the sublayer's output
+//   lay::postnorm_add      y = x + g * v / sqrt(mean(v^2) + eps): a branch's result is normed, then added
 //   lay::depth_mix         x = sum_j a[j] X_j over the stack of earlier layer results
 //   lay::route_sigmoid_topk, moe_group, moe_gather, moe_combine: sigmoid router whose score
 //                          scales the expert's input, rows grouped by expert for the grouped linear

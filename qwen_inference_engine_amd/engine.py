@@ -317,6 +317,12 @@ class Batch:
         _lib.check(self.lib.qie_batch_step_sample(self.h, C.byref(sc), out), "qie_batch_step_sample")
         return list(out)[:n]
 
+    def graph_stats(self):
+        """(instantiated step graphs, replays so far) of a layered batch."""
+        n, r = C.c_int32(), C.c_int64()
+        _lib.check(self.lib.qie_batch_step_graphs(self.h, C.byref(n), C.byref(r)), "qie_batch_step_graphs")
+        return n.value, r.value
+
     def keep_layers(self, on: bool = True) -> None:
         _lib.check(self.lib.qie_batch_keep_layers(self.h, int(on)), "qie_batch_keep_layers")
 

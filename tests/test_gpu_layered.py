@@ -306,6 +306,45 @@ def test_greedy_generation_through_the_batcher(model):
     assert cb.batch.page_stats()[0] == 8
 
 
+# ------------------------------------------------------------------ graph replays of small steps
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_small_steps_replay_graphs_equal_eager(dtype):
+    """Decoding steps of one shape are captured once and replayed; between the replays the
+    program does its own eager work (a prompt portion of another request, a release, a step of
+    another shape).  Every replayed step's logits equal the eager engine's bit for bit."""
+    a = Model(MIXED, seed=91, dtype=dtype)
+    b = Model(MIXED, seed=91, dtype=dtype)
+    b.batch.close()
+    b.eng.close()
+    import qwen_inference_engine_amd as q
+    b.eng = q.Engine(b.spec, max_ctx=512, dtype=dtype, use_graph=False).load_tensors({k: words(v) for k, v in b.T.items()})
+    b.batch = b.eng.batch(4, 512, page_tokens=16)
+    try:
+        toks = a.tokens(60)
+        other = a.tokens(40)
+        for m in (a, b):
+            m.out, m.tail = [m.batch.step([(0, toks[:20]), (1, other[:11])], [19, 30])], []
+            for i in range(20, 60):
+                if i % 7 == 0:                     # eager work between replays: another shape
+                    m.out.append(m.batch.step([(2, other[:5])], [4]))
+                    m.batch.release(2)
+                if i < 40:
+                    entries, want = [(0, [toks[i]]), (1, [other[i - 9]])], [0, 1]
+                else:                              # then single-row steps (a second graph)
+                    entries, want = [(0, [toks[i]])], [0]
+                m.out.append(m.batch.step(entries, want))
+                if i >= 40:
+                    m.tail.append(m.out[-1][0])
+        assert a.batch.graph_stats()[0] >= 2 and a.batch.graph_stats()[1] >= 30
+        assert b.batch.graph_stats() == (0, 0)
+        for x, y in zip(a.out, b.out):
+            assert np.array_equal(x, y)
+        assert (rel if dtype == "float32" else rel_most)(np.stack(a.tail), a.ref(toks)[40:60]) < a.tol
+    finally:
+        a.close()
+        b.close()
+
+
 # ------------------------------------------------------------------ the command-line programs
 def write_model_dir(path, cfg, T):
     """config.json + model.safetensors (8-byte header length, JSON header, bf16 data)."""
