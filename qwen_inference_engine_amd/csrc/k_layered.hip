@@ -239,7 +239,6 @@ static bool al16p(const void* q) { return ((uintptr_t)q & 15) == 0; }
 
 int linear(const LinearP& p, bool w_f32, hipStream_t st) {
     QIE_REQUIRE(p.A && p.W && p.Y && p.M > 0 && p.N > 0 && p.K > 0 && p.batch > 0, "layered linear: bad arguments");
-    const int esz = w_f32 ? 4 : 2;
     const bool a_vec = p.lda % 4 == 0 && p.sA % 4 == 0 && al16p(p.A);
     if (p.M <= 32) {
         const bool vec = a_vec && p.K % 8 == 0 && p.ldw % 8 == 0 && p.sW % 8 == 0 && al16p(p.W);
@@ -260,7 +259,6 @@ int linear(const LinearP& p, bool w_f32, hipStream_t st) {
         QIE_LAUNCH_CHECK();
         return 0;
     }
-    (void)esz;
     dim3 grid((unsigned)((p.N + LBN - 1) / LBN), (unsigned)((p.M + LBM - 1) / LBM), (unsigned)p.batch);
     if (w_f32)
         hipLaunchKernelGGL(linear_kernel<float>, grid, dim3(256), 0, st, p);

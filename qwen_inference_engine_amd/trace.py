@@ -73,6 +73,8 @@ def main(argv=None) -> int:
                 if not free:
                     raise RuntimeError(f"step {st['step']}: more than {SLOTS} live requests")
                 slot_of[rid] = free.pop()
+            if not en["tokens"]:                # admitted, nothing to run yet
+                continue
             entries.append((slot_of[rid], en["tokens"]))
             want += [row0 + int(w) for w in en.get("want", ())]
             row0 += len(en["tokens"])
