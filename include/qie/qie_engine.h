@@ -261,6 +261,8 @@ int qie_batch_debug_step(qie_batch* b, const qie_sampling* smp, int32_t* next_id
  * W_uv applied to the softmax-weighted sum of c), for prompts and decoding alike.
  * Feed-forward: none, dense gated SiLU, or a mixture of `experts` gated-SiLU experts with a
  * sigmoid router (fp32) whose `top` largest scores, not renormalised, scale the experts' input.
+ * (Ranked by the fp32 router logits, which order the experts as the scores do but do not
+ * saturate; equal logits: the lower index.)
  * Layer: y = x + g1 * rms(mixer(x)); z = y + g2 * rms(ff(y)) (scalar gains; each branch is
  * normed after it is computed, its input is the raw stream); the next layer's input is the depth-weighted sum over the embedding
  * output and every layer result so far. */

@@ -553,32 +553,34 @@ int silu_mul(const float* gu, float* a, uint16_t* a_bf, int64_t M, int ff, hipSt
 
 // ------------------------------------------------------------------ mixture of experts
 // Router: z = W_r y in fp32, s = sigmoid(z); the `top` largest (ties: the lower index) in
-// descending order -> sel[t, k], score[t, k].  One block per row.
+// descending order -> sel[t, k], score[t, k].  The ranking compares z, which orders the experts
+// as s does but does not saturate (sigmoid(z) is 1.0f for every z above ~17).  One block per row.
 template <typename TW>
 __global__ __launch_bounds__(256) void route_kernel(const float* y, const TW* Wr, int W, int E, int top, int32_t* sel,
                                                     float* score) {
-    extern __shared__ float s[];   // [E]
+    extern __shared__ float s[];   // [E] router logits
     const int64_t t = blockIdx.x;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     for (int e = wave; e < E; e += 4) {
         float z = 0.f;
         for (int i = lane; i < W; i += 64) z = fmaf(y[t * W + i], ldf<TW>(Wr, (int64_t)e * W + i), z);
         z = wave_sum(z);
-        if (lane == 0) s[e] = 1.0f / (1.0f + expf(-z));
+        if (lane == 0) s[e] = z;
     }
     __syncthreads();
     if (threadIdx.x == 0) {
         for (int k = 0; k < top; k++) {
-            int best = 0;
-            float bv = -1.f;
+            int best = -1;
+            float bv = 0.f;
             for (int e = 0; e < E; e++)
-                if (s[e] > bv) {
+                if (s[e] != -INFINITY && (best < 0 || s[e] > bv)) {
                     bv = s[e];
                     best = e;
                 }
+            if (best < 0) best = 0;   // only if logits are not finite
             sel[t * top + k] = best;
-            score[t * top + k] = bv;
-            s[best] = -2.f;
+            score[t * top + k] = 1.0f / (1.0f + expf(-bv));
+            s[best] = -INFINITY;
         }
     }
 }
