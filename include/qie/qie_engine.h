@@ -266,8 +266,55 @@ int qie_batch_debug_step(qie_batch* b, const qie_sampling* smp, int32_t* next_id
  * Layer: y = x + g1 * rms(mixer(x)); z = y + g2 * rms(ff(y)) (scalar gains; each branch is
  * normed after it is computed, its input is the raw stream); the next layer's input is the depth-weighted sum over the embedding
  * output and every layer result so far. */
-enum { QIE_MIXER_LATENT_ATTENTION = 1 };
+enum { QIE_MIXER_LATENT_ATTENTION = 1, QIE_MIXER_GQA = 2, QIE_MIXER_GQA_RECURRENT = 3 };
 enum { QIE_FF_NONE = 0, QIE_FF_DENSE = 1, QIE_FF_MOE = 2 };
+/* Which keys j <= i a query at position i sees: all of them; the last `size`; those of its own
+ * block of `size` positions (blocks counted from position 0 of the sequence). */
+enum { QIE_MASK_CAUSAL = 0, QIE_MASK_WINDOW = 1, QIE_MASK_CHUNK = 2 };
+/* RMS norm of every query / key head over dim before rotation: none, with a weight vector
+ * shared by the heads, or without one. */
+enum { QIE_QKNORM_NONE = 0, QIE_QKNORM_WEIGHT = 1, QIE_QKNORM_PLAIN = 2 };
+/* Rotary pairs inside the rotated coordinates: i with i + dims / 2, or 2i with 2i + 1. */
+enum { QIE_ROT_HALVES = 0, QIE_ROT_INTERLEAVED = 1 };
+/* Block: 0 = y = x + g * rms(branch(x)) with scalar gains (branches read the raw stream);
+ * 1 = x += N_b(branch(N_a(x))) with weight vectors stored around zero (N(v) = rms(v) (1 + w))
+ * before and after every branch. */
+enum { QIE_BLOCK_POSTNORM_GAIN = 0, QIE_BLOCK_SANDWICH = 1 };
+/* Router: 0 = sigmoid scores, the `top` largest scale the experts' input; 1 = logits with a
+ * bias, the `top` largest weighted by the softmax over those alone scale the experts' output. */
+enum { QIE_ROUTER_SIGMOID_IN = 0, QIE_ROUTER_SOFTMAX_OUT = 1 };
+
+/* Mixer QIE_MIXER_GQA: grouped-query softmax attention over a paged K / V cache.  q = W_q h
+ * (heads x dim), k = W_k h (kv_heads x dim), v = W_v h (kv_heads x vdim); query head h reads
+ * key / value head h / (heads / kv_heads).  Options, each a parameter: the q / k head norm; a
+ * rotary on the first rot_dims coordinates of q and k (angle pos * rot_base^(-2i / rot_dims));
+ * rot_values: the value at position j is turned by j over all vdim coordinates (same pairing,
+ * angle j * rot_base^(-2m / vdim)), cached so, and a head's weighted sum at position i is turned
+ * back by i; the mask; values_are_keys: no W_v, the value is the projected key as it leaves W_k
+ * (before its norm; vdim == dim); dist_bias: the score loses r1_h * ln(1 + r2_h * (i - j)). */
+typedef struct qie_gqa_desc {
+    int32_t heads, kv_heads, dim, vdim;
+    int32_t qk_norm;          /* QIE_QKNORM_*   */
+    int32_t rot_dims;         /* even, <= dim; 0 = no rotation of q and k */
+    int32_t rot_layout;       /* QIE_ROT_*      */
+    int32_t rot_values;
+    int32_t mask, mask_size;  /* QIE_MASK_*     */
+    int32_t values_are_keys;
+    int32_t dist_bias;
+    float rot_base, scale;
+    int32_t reserved[2];
+} qie_gqa_desc;
+
+/* Gated linear recurrence (the second half of QIE_MIXER_GQA_RECURRENT): per head a state
+ * S [dim][vdim] in fp32 that lives in the slot, S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T,
+ * o_t = S_t^T q_t with q = silu(W_q h), v = W_v h and the forget gate
+ * f = lower + (1 - lower) * sigmoid(W_f h + b); o is RMS-normed per head over vdim with a weight
+ * vector.  A slot that starts at position 0 starts from S = 0.  The mixer's result is
+ * gqa_scale * attention + rec_scale * recurrence (each after its own output projection). */
+typedef struct qie_recurrent_desc {
+    int32_t heads, dim, vdim;
+    int32_t reserved;
+} qie_recurrent_desc;
 
 typedef struct qie_layer_desc {
     int32_t mixer;            /* QIE_MIXER_*                                          */
@@ -279,21 +326,34 @@ typedef struct qie_layer_desc {
     int32_t ff_kind;          /* QIE_FF_*                                             */
     int32_t ff;               /* hidden size of the dense feed-forward / of one expert */
     int32_t experts, top;
-    int32_t reserved[4];
+    int32_t router;           /* QIE_ROUTER_*                                          */
+    int32_t reserved[3];
+    qie_gqa_desc gqa;         /* QIE_MIXER_GQA, QIE_MIXER_GQA_RECURRENT                */
+    qie_recurrent_desc rec;   /* QIE_MIXER_GQA_RECURRENT                               */
+    float gqa_scale, rec_scale;
 } qie_layer_desc;
 
 typedef struct qie_arch_desc {
     int32_t n_layers, width, vocab;
     float norm_eps;
     int32_t depth_mix;        /* 1: depth-weighted sum of all earlier results ('l<i>.dwa') */
-    int32_t reserved[7];
+    int32_t block;            /* QIE_BLOCK_*                                            */
+    int32_t tied_head;        /* 1: the logits are taken against 'embed' (no 'head')    */
+    /* layers [loop_start, loop_stop) run loop_times times in a row with the same weights (each
+     * run with its own cache region and state); before every run of the group but the first
+     * the embedding rows are added to the stream.  loop_times <= 1: every layer once. */
+    int32_t loop_start, loop_stop, loop_times;
+    int32_t reserved[2];
     const qie_layer_desc* layers;
 } qie_arch_desc;
 
 int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* opts, qie_engine** out);
 /* Hand the engine one checkpoint tensor (host memory, copied): dtype 0 = bf16 words, 1 = int32,
- * 2 = fp32.  Names: 'embed', 'head', 'final.norm', 'l<i>.norm1|norm2|dwa',
- * 'l<i>.mix.q|dkv|dkv.norm|uk|uv|g|o', 'l<i>.mlp.gate|up|down|router', 'l<i>.mlp.e<j>.gate|up|down'.
+ * 2 = fp32.  Names: 'embed', 'head', 'final.norm', 'l<i>.norm1|norm2|dwa' (sandwich blocks: also
+ * 'l<i>.norm1b|norm2b', all vectors of the width), 'l<i>.mix.q|dkv|dkv.norm|uk|uv|g|o' (latent
+ * attention), 'l<i>.mix.q|k|v|q.norm|k.norm|r1|r2|o' (QIE_MIXER_GQA; under 'l<i>.mix.left.' when a
+ * recurrence runs beside it, whose tensors are 'l<i>.mix.right.q|f|f.b|lower|v|norm|o'),
+ * 'l<i>.mlp.gate|up|down|router|router.b', 'l<i>.mlp.e<j>.gate|up|down'.
  * qie_engine_finalize_weights checks every tensor the architecture needs against its shape,
  * builds the device layouts (fused projection rows, per-head transposed W_uk, experts end to
  * end) and drops the host copies. */
@@ -318,13 +378,17 @@ int qie_batch_step_sample(qie_batch* b, const qie_sampling* s, int32_t* host_ids
  * per-step value (ids, slots, positions, block table, row groups) is read from device memory.
  * Instantiated graphs and replays so far: */
 int qie_batch_step_graphs(qie_batch* b, int32_t* n_graphs, int64_t* n_replays);
-/* Diagnostics: enable != 0 makes every following step keep the stream after each layer;
- * qie_batch_step_layers copies the last step's [n_layers][rows][width] fp32 to host_out. */
+/* Diagnostics: enable != 0 makes every following step keep the stream after each layer run (a
+ * repeated layer counts every time); qie_batch_step_layers copies the last step's
+ * [layer runs][rows][width] fp32 to host_out.  qie_engine_layer_runs: how many there are. */
+int qie_engine_layer_runs(const qie_engine* e);
 int qie_batch_keep_layers(qie_batch* b, int32_t enable);
 int qie_batch_step_layers(qie_batch* b, float* host_out, int64_t n);
 /* Time `iters` runs of one stage of the last step's shape (hipEvents on the engine stream):
  * which 0 = the whole layer stack, 1 = attention of `layer`, 2 = its projections (input, absorb,
- * value expansion, output), 3 = its feed-forward.  The cache is read, not advanced. */
+ * value expansion, output), 3 = its feed-forward, 4 = its gated recurrence (scan + head norm; the
+ * slots' states of that layer run are advanced by it, so time it last).  The cache is read, not
+ * advanced. */
 int qie_batch_time_stage(qie_batch* b, int32_t which, int32_t layer, int32_t iters, double* avg_us);
 
 #ifdef __cplusplus

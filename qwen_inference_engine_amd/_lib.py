@@ -81,8 +81,24 @@ class EngineOptsC(C.Structure):
                 ("compute_f32", C.c_int32), ("reserved", C.c_int32 * 4)]
 
 
-QIE_MIXER_LATENT_ATTENTION = 1
+QIE_MIXER_LATENT_ATTENTION, QIE_MIXER_GQA, QIE_MIXER_GQA_RECURRENT = 1, 2, 3
 QIE_FF_NONE, QIE_FF_DENSE, QIE_FF_MOE = 0, 1, 2
+QIE_MASK_CAUSAL, QIE_MASK_WINDOW, QIE_MASK_CHUNK = 0, 1, 2
+QIE_QKNORM_NONE, QIE_QKNORM_WEIGHT, QIE_QKNORM_PLAIN = 0, 1, 2
+QIE_ROT_HALVES, QIE_ROT_INTERLEAVED = 0, 1
+QIE_BLOCK_POSTNORM_GAIN, QIE_BLOCK_SANDWICH = 0, 1
+QIE_ROUTER_SIGMOID_IN, QIE_ROUTER_SOFTMAX_OUT = 0, 1
+
+
+class GqaDescC(C.Structure):
+    _fields_ = [("heads", C.c_int32), ("kv_heads", C.c_int32), ("dim", C.c_int32), ("vdim", C.c_int32),
+                ("qk_norm", C.c_int32), ("rot_dims", C.c_int32), ("rot_layout", C.c_int32), ("rot_values", C.c_int32),
+                ("mask", C.c_int32), ("mask_size", C.c_int32), ("values_are_keys", C.c_int32), ("dist_bias", C.c_int32),
+                ("rot_base", C.c_float), ("scale", C.c_float), ("reserved", C.c_int32 * 2)]
+
+
+class RecurrentDescC(C.Structure):
+    _fields_ = [("heads", C.c_int32), ("dim", C.c_int32), ("vdim", C.c_int32), ("reserved", C.c_int32)]
 
 
 class LayerDescC(C.Structure):
@@ -90,12 +106,15 @@ class LayerDescC(C.Structure):
                 ("vdim", C.c_int32), ("kv_rank", C.c_int32), ("window", C.c_int32), ("kv_from", C.c_int32),
                 ("rot_dims", C.c_int32), ("rot_base", C.c_float), ("scale", C.c_float),
                 ("ff_kind", C.c_int32), ("ff", C.c_int32), ("experts", C.c_int32), ("top", C.c_int32),
-                ("reserved", C.c_int32 * 4)]
+                ("router", C.c_int32), ("reserved", C.c_int32 * 3),
+                ("gqa", GqaDescC), ("rec", RecurrentDescC), ("gqa_scale", C.c_float), ("rec_scale", C.c_float)]
 
 
 class ArchDescC(C.Structure):
     _fields_ = [("n_layers", C.c_int32), ("width", C.c_int32), ("vocab", C.c_int32), ("norm_eps", C.c_float),
-                ("depth_mix", C.c_int32), ("reserved", C.c_int32 * 7), ("layers", C.POINTER(LayerDescC))]
+                ("depth_mix", C.c_int32), ("block", C.c_int32), ("tied_head", C.c_int32),
+                ("loop_start", C.c_int32), ("loop_stop", C.c_int32), ("loop_times", C.c_int32),
+                ("reserved", C.c_int32 * 2), ("layers", C.POINTER(LayerDescC))]
 
 
 # (name, restype, argtypes) — every symbol the public headers declare.
@@ -219,6 +238,7 @@ SIGNATURES = [
     ("qie_batch_step", C.c_int, [_P, _I32, _PI32, _PI32, _PI32, _I32, _PI32, _PF]),
     ("qie_batch_step_sample", C.c_int, [_P, C.POINTER(SamplingC), _PI32]),
     ("qie_batch_step_graphs", C.c_int, [_P, _PI32, _PI64]),
+    ("qie_engine_layer_runs", C.c_int, [_P]),
     ("qie_batch_keep_layers", C.c_int, [_P, _I32]),
     ("qie_batch_step_layers", C.c_int, [_P, _PF, _I64]),
     ("qie_batch_time_stage", C.c_int, [_P, _I32, _I32, _I32, _PD]),

@@ -2,8 +2,9 @@
 // (qie_engine_create_layered, qie_engine_put_tensor, qie_batch_step; qie_engine.h).
 //
 // A layered engine is a qie_engine whose `lm` holds the architecture and the device weights; a
-// batch of it is a paged qie_batch whose pool holds latent cache rows instead of K / V rows and
-// whose `lb` holds the step's activations.  Slots, the block table and the page pool are the
+// batch of it is a paged qie_batch whose pool holds, per layer run, the rows its mixer caches
+// (latent rows, or K and V rows of a grouped-query attention), whose `lb` holds the step's
+// activations and, for recurrent mixers, one fp32 state per slot and layer run.  Slots, the block table and the page pool are the
 // batch's own (ensure_pages / drop_pages / flush_table, qie_batch_release, qie_batch_page_stats).
 //
 // A step packs the rows of all entries (portions of prompts and single tokens alike) end to
@@ -55,6 +56,22 @@ struct LayerDev {
     void* w_down = nullptr;   // dense [width][ff];   moe [experts][width][ff]
     void* w_router = nullptr;
     float* dwa = nullptr;     // [i + 2]
+    // QIE_MIXER_GQA / QIE_MIXER_GQA_RECURRENT: w_in = [q ; k ; (v) ; rec q ; rec f ; rec v] rows,
+    // wo = [W_o of the attention | W_o of the recurrence] columns
+    int col_k = 0, col_v = -1, col_rq = 0, col_rf = 0, col_rv = 0, n_cat = 0, cat_rec = 0;
+    int rope_v = 0;
+    float *qn_w = nullptr, *kn_w = nullptr, *r1 = nullptr, *r2 = nullptr;
+    float *rec_fb = nullptr, *rec_lower = nullptr, *rec_norm = nullptr;
+    // sandwich blocks: weight vectors of the four norms; biased routers
+    float *n1 = nullptr, *n1b = nullptr, *n2 = nullptr, *n2b = nullptr;
+    float* router_b = nullptr;
+};
+
+// One execution of a layer: layers of a repeated group run several times, each run with its
+// own cache region and recurrent state.
+struct LayerRun {
+    int layer = 0;
+    bool add_embed = false;   // the embedding rows are added to the stream before this run
 };
 
 struct LayeredModel {
@@ -67,13 +84,28 @@ struct LayeredModel {
     void* embed = nullptr;
     void* head = nullptr;
     float g_final = 1.f;
+    float* w_final = nullptr;   // sandwich blocks: the output norm's weight vector
+    std::vector<LayerRun> runs;
+    bool loops = false;
     std::vector<void*> allocs;
     bool final = false;
     size_t esz() const { return f32 ? 4 : 2; }
 };
 
 struct LayeredBatch {
-    std::vector<int64_t> layer_off;   // element offset of each caching layer's rows inside a page
+    std::vector<int64_t> layer_off;   // per layer run: element offset of its (K) rows inside a page
+    std::vector<int64_t> v_off;       // per layer run: its V rows (grouped-query attention)
+    std::vector<int64_t> state_off;   // per layer run: its recurrent state inside a slot's state
+    float* state = nullptr;           // [slots][slot_state] fp32
+    int64_t slot_state = 0;
+    int4* d_ent = nullptr;            // the step's entries {first packed row, rows, slot, first position}
+    int64_t ent_cap = 0;
+    int n_ent = 0;
+    std::vector<int4> h_ent;
+    int4* d_qgroups = nullptr;        // matrix-core grouped-query attention: 16-row groups of the step's entries
+    int64_t qgroups_cap = 0;
+    int n_qgroups = 0;
+    std::vector<int4> h_qgroups;
     int64_t cap = 0, want_cap = 0;
     float *stack = nullptr, *x = nullptr, *proj = nullptr, *qabs = nullptr, *olat = nullptr, *ov = nullptr, *mix = nullptr,
           *y = nullptr, *gu = nullptr, *act = nullptr, *ffo = nullptr, *xg = nullptr, *yd = nullptr, *score = nullptr,
@@ -227,11 +259,103 @@ void layered_engine_destroy(qie_engine* e) {
     const HostTensor* var = lm_find(m, name, {__VA_ARGS__});     \
     if (!var) return -22
 
+// weight vector of a norm (sandwich blocks), length n
+static int lm_vector(LayeredModel* m, float** dev, const std::string& name, int64_t n) {
+    const HostTensor* t = lm_find(m, name, {n});
+    if (!t) return -22;
+    return lm_floats(m, dev, *t);
+}
+
+// Fused input rows and output columns of a grouped-query attention, alone ('mix.') or beside a
+// gated recurrence ('mix.left.' / 'mix.right.').
+static int finalize_gqa_mixer(qie_engine* e, LayeredModel* m, int i) {
+    LayerDev& L = m->L[i];
+    const qie_layer_desc& d = L.d;
+    const qie_gqa_desc& a = d.gqa;
+    const bool rec = d.mixer == QIE_MIXER_GQA_RECURRENT;
+    const int64_t W = m->a.width;
+    const std::string pl = "l" + std::to_string(i) + ".", pa = pl + (rec ? "mix.left." : "mix."), pr = pl + "mix.right.";
+    const int64_t nq = (int64_t)a.heads * a.dim, nk = (int64_t)a.kv_heads * a.dim, nv = a.values_are_keys ? 0 : (int64_t)a.kv_heads * a.vdim;
+    const int64_t rq = rec ? (int64_t)d.rec.heads * d.rec.dim : 0, rv = rec ? (int64_t)d.rec.heads * d.rec.vdim : 0;
+    L.col_k = (int)nq;
+    L.col_v = a.values_are_keys ? -1 : (int)(nq + nk);
+    L.col_rq = (int)(nq + nk + nv);
+    L.col_rf = (int)(L.col_rq + rq);
+    L.col_rv = (int)(L.col_rf + rq);
+    L.n_in = (int)(L.col_rv + rv);
+    QIE_TRY(lm_alloc(m, &L.w_in, (size_t)L.n_in * W * m->esz()));
+    LM_GET(tq, pa + "q", nq, W);
+    LM_GET(tk, pa + "k", nk, W);
+    QIE_TRY(lm_upload_rows(m, L.w_in, 0, W, *tq));
+    QIE_TRY(lm_upload_rows(m, L.w_in, L.col_k, W, *tk));
+    if (!a.values_are_keys) {
+        LM_GET(tv, pa + "v", nv, W);
+        QIE_TRY(lm_upload_rows(m, L.w_in, L.col_v, W, *tv));
+    }
+    if (a.qk_norm == QIE_QKNORM_WEIGHT) {
+        QIE_TRY(lm_vector(m, &L.qn_w, pa + "q.norm", a.dim));
+        QIE_TRY(lm_vector(m, &L.kn_w, pa + "k.norm", a.dim));
+    }
+    if (a.dist_bias) {
+        QIE_TRY(lm_vector(m, &L.r1, pa + "r1", a.heads));
+        QIE_TRY(lm_vector(m, &L.r2, pa + "r2", a.heads));
+    }
+    if (a.rot_dims > 0) QIE_TRY(lm_rope(m, e, (double)a.rot_base, a.rot_dims, &L.rope));
+    if (a.rot_values) QIE_TRY(lm_rope(m, e, (double)a.rot_base, a.vdim, &L.rope_v));
+    const int64_t ca = (int64_t)a.heads * a.vdim;
+    L.cat_rec = (int)ca;
+    L.n_cat = (int)(ca + rv);
+    QIE_TRY(lm_alloc(m, &L.wo, (size_t)W * L.n_cat * m->esz()));
+    LM_GET(to, pa + "o", W, ca);
+    if (!rec) {
+        QIE_TRY(lm_upload_rows(m, L.wo, 0, ca, *to));
+        return 0;
+    }
+    LM_GET(trq, pr + "q", rq, W);
+    LM_GET(trf, pr + "f", rq, W);
+    LM_GET(trv, pr + "v", rv, W);
+    QIE_TRY(lm_upload_rows(m, L.w_in, L.col_rq, W, *trq));
+    QIE_TRY(lm_upload_rows(m, L.w_in, L.col_rf, W, *trf));
+    QIE_TRY(lm_upload_rows(m, L.w_in, L.col_rv, W, *trv));
+    QIE_TRY(lm_vector(m, &L.rec_fb, pr + "f.b", rq));
+    QIE_TRY(lm_vector(m, &L.rec_lower, pr + "lower", rq));
+    QIE_TRY(lm_vector(m, &L.rec_norm, pr + "norm", d.rec.vdim));
+    LM_GET(tro, pr + "o", W, rv);
+    {   // [W][ca] and [W][rv] side by side: one product over the concatenated head outputs
+        HostTensor cat;
+        cat.dtype = 2;
+        cat.shape = {W, (int64_t)L.n_cat};
+        cat.data.resize((size_t)W * L.n_cat * 4);
+        float* c = (float*)cat.data.data();
+        for (int64_t r = 0; r < W; r++) {
+            for (int64_t k = 0; k < ca; k++) c[r * L.n_cat + k] = host_elem(*to, r * ca + k);
+            for (int64_t k = 0; k < rv; k++) c[r * L.n_cat + ca + k] = host_elem(*tro, r * rv + k);
+        }
+        QIE_TRY(lm_upload_rows(m, L.wo, 0, L.n_cat, cat));
+    }
+    return 0;
+}
+
+static int finalize_ff(LayeredModel* m, int i);
+
 static int finalize_layer(qie_engine* e, LayeredModel* m, int i) {
     LayerDev& L = m->L[i];
     const qie_layer_desc& d = L.d;
-    const int64_t W = m->a.width, H = d.heads, hq = d.dim + d.rot_dim, R = d.kv_rank;
     const std::string pl = "l" + std::to_string(i) + ".", px = pl + "mix.";
+    if (m->a.block == QIE_BLOCK_SANDWICH) {
+        const int64_t Wn = m->a.width;
+        QIE_TRY(lm_vector(m, &L.n1, pl + "norm1", Wn));
+        QIE_TRY(lm_vector(m, &L.n1b, pl + "norm1b", Wn));
+        if (d.ff_kind != QIE_FF_NONE) {
+            QIE_TRY(lm_vector(m, &L.n2, pl + "norm2", Wn));
+            QIE_TRY(lm_vector(m, &L.n2b, pl + "norm2b", Wn));
+        }
+    }
+    if (d.mixer != QIE_MIXER_LATENT_ATTENTION) {
+        QIE_TRY(finalize_gqa_mixer(e, m, i));
+        return finalize_ff(m, i);
+    }
+    const int64_t W = m->a.width, H = d.heads, hq = d.dim + d.rot_dim, R = d.kv_rank;
     const bool own = d.kv_from < 0;
     LM_GET(tq, px + "q", H * hq, W);
     LM_GET(tg, px + "g", H, W);
@@ -262,13 +386,28 @@ static int finalize_layer(qie_engine* e, LayeredModel* m, int i) {
     LM_GET(to, px + "o", W, H * d.vdim);
     QIE_TRY(lm_alloc(m, &L.wo, (size_t)to->numel() * m->esz()));
     QIE_TRY(lm_upload_rows(m, L.wo, 0, H * d.vdim, *to));
-    LM_GET(n1, pl + "norm1");
-    L.g1 = host_elem(*n1, 0);
     QIE_TRY(lm_rope(m, e, (double)d.rot_base, d.rot_dims, &L.rope));
-    if (d.ff_kind != QIE_FF_NONE) {
-        LM_GET(n2, pl + "norm2");
-        L.g2 = host_elem(*n2, 0);
+    if (m->a.block == QIE_BLOCK_POSTNORM_GAIN) {
+        LM_GET(n1, pl + "norm1");
+        L.g1 = host_elem(*n1, 0);
+        if (d.ff_kind != QIE_FF_NONE) {
+            LM_GET(n2, pl + "norm2");
+            L.g2 = host_elem(*n2, 0);
+        }
     }
+    QIE_TRY(finalize_ff(m, i));
+    if (m->a.depth_mix) {
+        LM_GET(da, pl + "dwa", (int64_t)i + 2);
+        QIE_TRY(lm_floats(m, &L.dwa, *da));
+    }
+    return 0;
+}
+
+static int finalize_ff(LayeredModel* m, int i) {
+    LayerDev& L = m->L[i];
+    const qie_layer_desc& d = L.d;
+    const int64_t W = m->a.width;
+    const std::string pl = "l" + std::to_string(i) + ".";
     const int64_t ff = d.ff;
     if (d.ff_kind == QIE_FF_DENSE) {
         LM_GET(wg, pl + "mlp.gate", ff, W);
@@ -284,6 +423,7 @@ static int finalize_layer(qie_engine* e, LayeredModel* m, int i) {
         LM_GET(wr, pl + "mlp.router", E, W);
         QIE_TRY(lm_alloc(m, &L.w_router, (size_t)E * W * m->esz()));
         QIE_TRY(lm_upload_rows(m, L.w_router, 0, W, *wr));
+        if (d.router == QIE_ROUTER_SOFTMAX_OUT) QIE_TRY(lm_vector(m, &L.router_b, pl + "mlp.router.b", E));
         QIE_TRY(lm_alloc(m, &L.w_gu, (size_t)E * 2 * ff * W * m->esz()));
         QIE_TRY(lm_alloc(m, &L.w_down, (size_t)E * W * ff * m->esz()));
         for (int64_t x = 0; x < E; x++) {
@@ -295,10 +435,6 @@ static int finalize_layer(qie_engine* e, LayeredModel* m, int i) {
             QIE_TRY(lm_upload_rows(m, L.w_gu, x * 2 * ff + ff, W, *wu));
             QIE_TRY(lm_upload_rows(m, L.w_down, x * W, ff, *wd));
         }
-    }
-    if (m->a.depth_mix) {
-        LM_GET(da, pl + "dwa", (int64_t)i + 2);
-        QIE_TRY(lm_floats(m, &L.dwa, *da));
     }
     return 0;
 }
@@ -377,7 +513,7 @@ static int enq_latent_post(qie_batch* b, int i, int T) {
     p.rope_cos = m->ropes[L.rope].cs;
     p.rope_sin = m->ropes[L.rope].sn;
     p.cache = cache_of(b);
-    p.layer_off = s->layer_off[L.cache_layer];
+    p.layer_off = s->layer_off[L.cache_layer];   // engines with latent layers run every layer once: run == layer
     p.interleaved = s->interleaved;
     return lay::latent_post(p, m->f32, T, e->stream);
 }
@@ -520,10 +656,13 @@ static int enq_ff(qie_batch* b, int i, int T) {
         return dense(b, s->act, ff, L.w_down, s->ffo, W, T, W, ff, s->act_bf);
     }
     const int E = d.experts, top = d.top, n = T * top;
-    QIE_TRY(lay::route_sigmoid_topk(s->y, L.w_router, m->f32, T, W, E, top, s->sel, s->score, st));
+    const bool out_w = d.router == QIE_ROUTER_SOFTMAX_OUT;   // the scores weight the outputs, not the inputs
+    const float* in_score = out_w ? nullptr : s->score;
+    const float* out_score = out_w ? s->score : nullptr;
+    QIE_TRY(lay::route_topk(s->y, L.w_router, L.router_b, m->f32, T, W, E, top, out_w ? 1 : 0, s->sel, s->score, st));
     QIE_TRY(lay::moe_group(s->sel, n, E, s->cnt, s->off, s->slot_of, st));
     const bool per_expert = !m->f32 && n >= kMoeSyncRows && W % 8 == 0 && ff % 8 == 0;
-    QIE_TRY(lay::moe_gather(s->y, s->score, s->slot_of, T, top, W, s->xg, per_expert ? s->xg_bf : nullptr, st));
+    QIE_TRY(lay::moe_gather(s->y, in_score, s->slot_of, T, top, W, s->xg, per_expert ? s->xg_bf : nullptr, st));
     if (per_expert) {
         // prompt-sized steps: the expert row ranges come to the host and every expert's rows go
         // through the MFMA kernels; the products are the grouped kernel's, in another order
@@ -564,12 +703,147 @@ static int enq_ff(qie_batch* b, int i, int T) {
                                  lane_of(x)));
         }
         QIE_TRY(join());
-        return lay::moe_combine(s->yd, s->slot_of, T, top, W, s->ffo, st);
+        return lay::moe_combine(s->yd, s->slot_of, out_score, T, top, W, s->ffo, st);
     }
     QIE_TRY(lin(e, s->xg, W, L.w_gu, W, s->gu, 2 * ff, n, 2 * ff, W, E, 0, (int64_t)2 * ff * W, 0, s->off));
     QIE_TRY(lay::silu_mul(s->gu, s->act, nullptr, n, ff, st));
     QIE_TRY(lin(e, s->act, ff, L.w_down, ff, s->yd, W, n, W, ff, E, 0, (int64_t)W * ff, 0, s->off));
-    return lay::moe_combine(s->yd, s->slot_of, T, top, W, s->ffo, st);
+    return lay::moe_combine(s->yd, s->slot_of, out_score, T, top, W, s->ffo, st);
+}
+
+// ---- grouped-query attention (+ gated recurrence) of layer run r; the branch input is s->y
+static lay::GqaAttnP gqa_attn_params(qie_batch* b, int r) {
+    const LayeredModel* m = b->e->lm;
+    const LayerDev& L = m->L[m->runs[r].layer];
+    const qie_gqa_desc& a = L.d.gqa;
+    LayeredBatch* s = b->lb;
+    lay::GqaAttnP p{};
+    p.proj = s->proj; p.ld = L.n_in; p.q_col = 0;
+    p.row_slot = s->row_slot; p.row_pos = s->row_pos;
+    p.heads = a.heads; p.kv_heads = a.kv_heads; p.dim = a.dim; p.vdim = a.vdim;
+    p.mask = a.mask; p.mask_size = a.mask_size; p.scale = a.scale;
+    p.r1 = a.dist_bias ? L.r1 : nullptr;
+    p.r2 = a.dist_bias ? L.r2 : nullptr;
+    p.rot_values = a.rot_values; p.rot_layout = a.rot_layout;
+    if (a.rot_values) {
+        p.vrope_cos = m->ropes[L.rope_v].cs;
+        p.vrope_sin = m->ropes[L.rope_v].sn;
+    }
+    p.cache = cache_of(b);
+    p.k_off = s->layer_off[r];
+    p.v_off = s->v_off[r];
+    p.out_scale = L.d.mixer == QIE_MIXER_GQA_RECURRENT ? L.d.gqa_scale : 1.0f;
+    p.out = s->ov; p.out_bf = s->ov_bf; p.ld_out = L.n_cat; p.out_col = 0;
+    return p;
+}
+
+static int enq_gqa_proj(qie_batch* b, int r, int T) {
+    const LayeredModel* m = b->e->lm;
+    const LayerDev& L = m->L[m->runs[r].layer];
+    LayeredBatch* s = b->lb;
+    return dense(b, s->y, m->a.width, L.w_in, s->proj, L.n_in, T, L.n_in, m->a.width, s->y_bf);
+}
+
+static int enq_gqa_post(qie_batch* b, int r, int T) {
+    const qie_engine* e = b->e;
+    const LayeredModel* m = e->lm;
+    const LayerDev& L = m->L[m->runs[r].layer];
+    const qie_gqa_desc& a = L.d.gqa;
+    LayeredBatch* s = b->lb;
+    lay::GqaPostP p{};
+    p.proj = s->proj; p.ld = L.n_in; p.q_col = 0; p.k_col = L.col_k; p.v_col = L.col_v;
+    p.row_slot = s->row_slot; p.row_pos = s->row_pos;
+    p.heads = a.heads; p.kv_heads = a.kv_heads; p.dim = a.dim; p.vdim = a.vdim;
+    p.qk_norm = a.qk_norm; p.qn_w = L.qn_w; p.kn_w = L.kn_w; p.eps = m->a.norm_eps;
+    p.rot_dims = a.rot_dims; p.rot_layout = a.rot_layout;
+    if (a.rot_dims > 0) {
+        p.rope_cos = m->ropes[L.rope].cs;
+        p.rope_sin = m->ropes[L.rope].sn;
+    }
+    p.rot_values = a.rot_values;
+    if (a.rot_values) {
+        p.vrope_cos = m->ropes[L.rope_v].cs;
+        p.vrope_sin = m->ropes[L.rope_v].sn;
+    }
+    p.cache = cache_of(b);
+    p.k_off = s->layer_off[r];
+    p.v_off = s->v_off[r];
+    return lay::gqa_post(p, m->f32, T, e->stream);
+}
+
+static int enq_gqa_attention(qie_batch* b, int r, int T) {
+    const qie_engine* e = b->e;
+    LayeredBatch* s = b->lb;
+    const lay::GqaAttnP p = gqa_attn_params(b, r);
+    if (!e->lm->f32 && s->n_qgroups > 0 && lay::gqa_attention_mfma_fits(p.dim, p.vdim)) {
+        lay::GqaAttnMfmaP q{p, s->d_qgroups, s->n_qgroups};
+        return lay::gqa_attention_mfma(q, e->stream);
+    }
+    return lay::gqa_attention(p, e->lm->f32, T, e->stream);
+}
+
+static int enq_recurrence(qie_batch* b, int r, int T) {
+    const qie_engine* e = b->e;
+    const LayeredModel* m = e->lm;
+    const LayerDev& L = m->L[m->runs[r].layer];
+    const qie_recurrent_desc& c = L.d.rec;
+    LayeredBatch* s = b->lb;
+    lay::GatedScanP p{};
+    p.proj = s->proj; p.ld = L.n_in; p.q_col = L.col_rq; p.f_col = L.col_rf; p.v_col = L.col_rv;
+    p.entries = s->d_ent; p.n_entries = s->n_ent;
+    p.heads = c.heads; p.dim = c.dim; p.vdim = c.vdim;
+    p.f_bias = L.rec_fb; p.lower = L.rec_lower;
+    p.state = s->state; p.slot_stride = s->slot_state; p.state_off = s->state_off[r];
+    p.out = s->olat;
+    QIE_TRY(lay::gated_scan(p, e->stream));
+    return lay::head_norm_rows(s->olat, L.rec_norm, m->a.norm_eps, L.d.rec_scale, c.heads, c.vdim, T, s->ov, s->ov_bf, L.n_cat,
+                               L.cat_rec, e->stream);
+}
+
+static int enq_gqa_mixer(qie_batch* b, int r, int T) {
+    const LayeredModel* m = b->e->lm;
+    const LayerDev& L = m->L[m->runs[r].layer];
+    LayeredBatch* s = b->lb;
+    QIE_TRY(enq_gqa_proj(b, r, T));
+    QIE_TRY(enq_gqa_post(b, r, T));
+    QIE_TRY(enq_gqa_attention(b, r, T));
+    if (L.d.mixer == QIE_MIXER_GQA_RECURRENT) QIE_TRY(enq_recurrence(b, r, T));
+    return dense(b, s->ov, L.n_cat, L.wo, s->mix, m->a.width, T, m->a.width, L.n_cat, s->ov_bf);
+}
+
+// Sandwich blocks: the stream x lives in plane 1 of the stack, the embedding rows stay in plane
+// 0.  h_ready: the run's normed input is already in s->y (the previous run's last kernel made
+// it).  The last kernel of the run also makes the next run's input unless the streams are kept.
+static int enq_run_sandwich(qie_batch* b, int r, int T, bool h_ready, bool* next_ready) {
+    const qie_engine* e = b->e;
+    const LayeredModel* m = e->lm;
+    const LayerDev& L = m->L[m->runs[r].layer];
+    LayeredBatch* s = b->lb;
+    const int W = m->a.width;
+    hipStream_t st = e->stream;
+    const int64_t plane = s->cap * W;
+    float* x0 = s->stack;
+    float* x = s->stack + plane;
+    const float eps = m->a.norm_eps;
+    if (!h_ready) QIE_TRY(lay::add_norm(x, x, nullptr, nullptr, m->runs[r].add_embed ? x0 : nullptr, L.n1, s->y, s->y_bf, T, W, eps, st));
+    QIE_REQUIRE(L.d.mixer != QIE_MIXER_LATENT_ATTENTION, "sandwich blocks: latent attention is not wired to them");
+    QIE_TRY(enq_gqa_mixer(b, r, T));
+    const bool has_ff = L.d.ff_kind != QIE_FF_NONE;
+    const bool last = r + 1 == (int)m->runs.size();
+    const bool fuse_next = !last && !s->keep_on;
+    const LayerDev* N = last ? nullptr : &m->L[m->runs[r + 1].layer];
+    const float* nx_add = fuse_next && m->runs[r + 1].add_embed ? x0 : nullptr;
+    if (has_ff) {
+        QIE_TRY(lay::add_norm(x, x, s->mix, L.n1b, nullptr, L.n2, s->y, s->y_bf, T, W, eps, st));
+        QIE_TRY(enq_ff(b, m->runs[r].layer, T));
+        QIE_TRY(lay::add_norm(x, x, s->ffo, L.n2b, nx_add, fuse_next ? N->n1 : nullptr, s->y, s->y_bf, T, W, eps, st));
+    } else {
+        QIE_TRY(lay::add_norm(x, x, s->mix, L.n1b, nx_add, fuse_next ? N->n1 : nullptr, s->y, s->y_bf, T, W, eps, st));
+    }
+    *next_ready = fuse_next;
+    if (s->keep_on && s->keep)
+        QIE_HIP(hipMemcpyAsync(s->keep + (int64_t)r * plane, x, (size_t)T * W * 4, hipMemcpyDeviceToDevice, st));
+    return 0;
 }
 
 static int enq_layer(qie_batch* b, int i, const float* xin, const uint16_t* xin_bf, int T, const float** xout,
@@ -611,12 +885,24 @@ static int enq_forward(qie_batch* b, int T, int n_want) {
     const LayeredModel* m = e->lm;
     LayeredBatch* s = b->lb;
     const int W = m->a.width;
-    QIE_TRY(lay::embed_rows(m->embed, m->f32, s->tok, s->stack, s->x_bf, T, W, m->a.vocab, e->stream));
     const float* x = s->stack;
-    const uint16_t* x_bf = s->x_bf;
-    for (int i = 0; i < m->a.n_layers; i++) QIE_TRY(enq_layer(b, i, x, x_bf, T, &x, &x_bf));
+    if (m->a.block == QIE_BLOCK_SANDWICH) {
+        // the embedding rows stay in plane 0 only when a repeated group adds them again
+        float* xs = s->stack + s->cap * W;
+        QIE_TRY(lay::embed_rows(m->embed, m->f32, s->tok, m->loops ? s->stack : xs, nullptr, T, W, m->a.vocab, e->stream));
+        const LayerDev& L0 = m->L[m->runs[0].layer];
+        QIE_TRY(lay::add_norm(xs, m->loops ? s->stack : xs, nullptr, nullptr, nullptr, L0.n1, s->y, s->y_bf, T, W, m->a.norm_eps,
+                              e->stream));
+        bool ready = true;
+        for (int r = 0; r < (int)m->runs.size(); r++) QIE_TRY(enq_run_sandwich(b, r, T, ready, &ready));
+        x = xs;
+    } else {
+        QIE_TRY(lay::embed_rows(m->embed, m->f32, s->tok, s->stack, s->x_bf, T, W, m->a.vocab, e->stream));
+        const uint16_t* x_bf = s->x_bf;
+        for (int i = 0; i < m->a.n_layers; i++) QIE_TRY(enq_layer(b, i, x, x_bf, T, &x, &x_bf));
+    }
     if (n_want > 0) {
-        QIE_TRY(lay::final_rows(x, s->want, s->xn, s->xn_bf, n_want, W, m->g_final, m->a.norm_eps, e->stream));
+        QIE_TRY(lay::final_rows(x, s->want, s->xn, s->xn_bf, n_want, W, m->g_final, m->w_final, m->a.norm_eps, e->stream));
         QIE_TRY(dense(b, s->xn, W, m->head, s->logits, m->a.vocab, n_want, m->a.vocab, W, s->xn_bf));
     }
     return 0;
@@ -653,7 +939,7 @@ static int run_forward(qie_batch* b, int T, int n_want) {
     for (const LayerDev& L : m->L)
         if (L.d.ff_kind == QIE_FF_MOE && (int64_t)T * L.d.top >= kMoeSyncRows) can = false;   // host round trip inside
     if (!can) return enq_forward(b, T, n_want);
-    std::vector<int> key{T, n_want};
+    std::vector<int> key{T, n_want, s->n_ent, s->n_qgroups};
     for (const auto& g : s->groups) {
         key.push_back(g.first);
         key.push_back(g.second.first);
@@ -701,7 +987,7 @@ static int ensure_rows(qie_batch* b, int64_t T) {
         auto A = [&](void** p, int64_t elems, size_t sz = 4) {
             if (!rc) rc = dmalloc(p, (size_t)elems * sz);
         };
-        A((void**)&s->stack, (L + 1) * cap * W);
+        A((void**)&s->stack, (m->a.depth_mix ? L + 1 : 2) * cap * W);
         A((void**)&s->x, cap * W);
         A((void**)&s->proj, cap * s->m_in);
         A((void**)&s->qabs, cap * s->m_hr);
@@ -730,12 +1016,12 @@ static int ensure_rows(qie_batch* b, int64_t T) {
             A((void**)&s->act_bf, cap * std::max<int64_t>(s->m_act, 1), 2);
             A((void**)&s->xg_bf, cap * std::max<int64_t>(s->m_top, 1) * W, 2);
         }
-        if (s->keep_on) A((void**)&s->keep, L * cap * W);
+        if (s->keep_on) A((void**)&s->keep, (int64_t)m->runs.size() * cap * W);
         if (rc) return rc;
         s->cap = cap;
     }
     if (s->keep_on && !s->keep) drop_graphs(s);
-    if (s->keep_on && !s->keep) QIE_TRY(dmalloc((void**)&s->keep, (size_t)m->a.n_layers * s->cap * m->a.width * 4));
+    if (s->keep_on && !s->keep) QIE_TRY(dmalloc((void**)&s->keep, m->runs.size() * s->cap * m->a.width * 4));
     if (T > s->h_stage_rows) {
         if (s->h_stage) hipHostFree(s->h_stage);
         s->h_stage = nullptr;
@@ -791,15 +1077,54 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
     b->page_tokens = page_tokens;
     b->max_pages = (max_ctx + page_tokens - 1) / page_tokens;
     b->n_pages = n_pages > 0 ? n_pages : batch * b->max_pages + 1;
-    s->layer_off.assign(m->a.n_layers, 0);
+    const int n_runs = (int)m->runs.size();
+    s->layer_off.assign(n_runs, 0);
+    s->v_off.assign(n_runs, 0);
+    s->state_off.assign(n_runs, 0);
     // bf16 caches whose every layer fits the matrix-core attention carry, after the rows of a
     // caching layer, the key-interleaved copy of c (R more elements per token)
     s->interleaved = !m->f32;
     for (int i = 0; i < m->a.n_layers; i++)
-        if (!lay::latent_attention_mfma_fits(m->L[i].d.kv_rank, m->L[i].d.rot_dim)) s->interleaved = false;
+        if (m->L[i].d.mixer != QIE_MIXER_LATENT_ATTENTION ||
+            !lay::latent_attention_mfma_fits(m->L[i].d.kv_rank, m->L[i].d.rot_dim))
+            s->interleaved = false;
     int64_t off = 0;
+    for (int r = 0; r < n_runs; r++) {
+        const int i = m->runs[r].layer;
+        const qie_layer_desc& d = m->L[i].d;
+        if (d.mixer != QIE_MIXER_LATENT_ATTENTION) {
+            // K rows, then V rows of this run; one state per slot for the recurrence
+            const qie_gqa_desc& a = d.gqa;
+            s->layer_off[r] = off;
+            off += (int64_t)page_tokens * a.kv_heads * a.dim;
+            s->v_off[r] = off;
+            off += (int64_t)page_tokens * a.kv_heads * a.vdim;
+            const int64_t rv = d.mixer == QIE_MIXER_GQA_RECURRENT ? (int64_t)d.rec.heads * d.rec.vdim : 0;
+            if (rv) {
+                s->state_off[r] = s->slot_state;
+                s->slot_state += (int64_t)d.rec.heads * d.rec.dim * d.rec.vdim;
+            }
+            s->m_in = std::max<int64_t>(s->m_in, m->L[i].n_in);
+            s->m_hr = std::max<int64_t>(s->m_hr, rv);
+            s->m_hv = std::max<int64_t>(s->m_hv, m->L[i].n_cat);
+            s->m_abf = std::max<int64_t>({s->m_abf, (int64_t)m->a.width, (int64_t)m->L[i].n_cat});
+        }
+    }
     for (int i = 0; i < m->a.n_layers; i++) {
         const qie_layer_desc& d = m->L[i].d;
+        const int64_t k = d.ff_kind == QIE_FF_MOE ? d.top : 1;
+        if (d.mixer != QIE_MIXER_LATENT_ATTENTION) {
+            if (d.ff_kind != QIE_FF_NONE) {
+                s->m_gu = std::max<int64_t>(s->m_gu, k * 2 * d.ff);
+                s->m_act = std::max<int64_t>(s->m_act, k * d.ff);
+                s->m_abf = std::max<int64_t>(s->m_abf, k * std::max<int64_t>(d.ff, m->a.width));
+            }
+            if (d.ff_kind == QIE_FF_MOE) {
+                s->m_top = std::max<int64_t>(s->m_top, d.top);
+                s->m_e = std::max<int64_t>(s->m_e, d.experts);
+            }
+            continue;
+        }
         if (d.kv_from < 0) {
             s->layer_off[i] = off;
             off += (int64_t)page_tokens * (d.kv_rank + d.rot_dim + (s->interleaved ? d.kv_rank : 0));
@@ -809,7 +1134,6 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
         s->m_hr = std::max<int64_t>(s->m_hr, H * d.kv_rank);
         s->m_r = std::max<int64_t>(s->m_r, d.kv_rank);
         s->m_hv = std::max<int64_t>(s->m_hv, H * d.vdim);
-        const int64_t k = d.ff_kind == QIE_FF_MOE ? d.top : 1;
         if (d.ff_kind != QIE_FF_NONE) {
             s->m_gu = std::max<int64_t>(s->m_gu, k * 2 * d.ff);
             s->m_act = std::max<int64_t>(s->m_act, k * d.ff);
@@ -831,8 +1155,10 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
     const size_t pool = (size_t)b->n_pages * off * m->esz();
     int rc = dmalloc((void**)&b->kc, pool);
     if (!rc) rc = dmalloc((void**)&b->d_table, b->h_table.size() * 4);
+    if (!rc && s->slot_state > 0) rc = dmalloc((void**)&s->state, (size_t)batch * s->slot_state * 4);
     if (!rc) {
         hipError_t he = hipMemsetAsync(b->kc, 0, pool, e->stream);
+        if (he == hipSuccess && s->state) he = hipMemsetAsync(s->state, 0, (size_t)batch * s->slot_state * 4, e->stream);
         if (he == hipSuccess) he = hipStreamSynchronize(e->stream);
         if (he != hipSuccess) rc = fail((int)he, "batch init: %s", hipGetErrorString(he));
     }
@@ -857,7 +1183,8 @@ void layered_batch_destroy(qie_batch* b) {
     LayeredBatch* s = b->lb;
     if (!s) return;
     lb_free(s);
-    void* ps[] = {s->want, s->xn, s->logits, s->logits_bf, s->d_ids, s->d_step, s->d_groups, s->part_o, s->part_ml, s->xn_bf};
+    void* ps[] = {s->want, s->xn, s->logits, s->logits_bf, s->d_ids, s->d_step, s->d_groups, s->part_o, s->part_ml, s->xn_bf,
+                  s->state, s->d_ent, s->d_qgroups};
     for (void* p : ps)
         if (p) hipFree(p);
     if (s->h_stage) hipHostFree(s->h_stage);
@@ -883,9 +1210,43 @@ int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* 
                 "qie_engine_create_layered: invalid sizes");
     QIE_REQUIRE(!opts || !opts->tp_comm, "qie_engine_create_layered: layered engines run on one device");
     QIE_REQUIRE(!opts || (!opts->weight_fp8 && !opts->prefill_fp8), "qie_engine_create_layered: fp8 weights are not covered");
+    QIE_REQUIRE(arch->block == QIE_BLOCK_POSTNORM_GAIN || arch->block == QIE_BLOCK_SANDWICH, "qie_engine_create_layered: block %d",
+                arch->block);
+    QIE_REQUIRE(arch->block == QIE_BLOCK_POSTNORM_GAIN || !arch->depth_mix,
+                "qie_engine_create_layered: depth-weighted residuals go with the post-norm block");
+    const bool loops = arch->loop_times > 1 && arch->loop_stop > arch->loop_start;
+    QIE_REQUIRE(!loops || (arch->loop_start >= 0 && arch->loop_stop <= arch->n_layers && arch->loop_times <= 64),
+                "qie_engine_create_layered: repeated group [%d, %d) x %d of %d layers", arch->loop_start, arch->loop_stop,
+                arch->loop_times, arch->n_layers);
+    QIE_REQUIRE(!loops || arch->block == QIE_BLOCK_SANDWICH, "qie_engine_create_layered: repeated groups go with the sandwich block");
     for (int i = 0; i < arch->n_layers; i++) {
         const qie_layer_desc& d = arch->layers[i];
+        QIE_REQUIRE(d.ff_kind >= QIE_FF_NONE && d.ff_kind <= QIE_FF_MOE, "layer %d: unknown feed-forward %d", i, d.ff_kind);
+        QIE_REQUIRE(d.ff_kind == QIE_FF_NONE || d.ff > 0, "layer %d: feed-forward size", i);
+        QIE_REQUIRE(d.ff_kind != QIE_FF_MOE || (d.experts > 0 && d.top > 0 && d.top <= d.experts), "layer %d: %d of %d experts", i,
+                    d.top, d.experts);
+        QIE_REQUIRE(d.router == QIE_ROUTER_SIGMOID_IN || d.router == QIE_ROUTER_SOFTMAX_OUT, "layer %d: router %d", i, d.router);
+        if (d.mixer == QIE_MIXER_GQA || d.mixer == QIE_MIXER_GQA_RECURRENT) {
+            const qie_gqa_desc& a = d.gqa;
+            QIE_REQUIRE(arch->block == QIE_BLOCK_SANDWICH, "layer %d: this mixer is wired to the sandwich block", i);
+            QIE_REQUIRE(a.heads > 0 && a.kv_heads > 0 && a.heads % a.kv_heads == 0 && a.dim > 0 && a.vdim > 0,
+                        "layer %d: %d query heads over %d key heads of %d / %d", i, a.heads, a.kv_heads, a.dim, a.vdim);
+            QIE_REQUIRE(a.qk_norm >= QIE_QKNORM_NONE && a.qk_norm <= QIE_QKNORM_PLAIN, "layer %d: q / k norm %d", i, a.qk_norm);
+            QIE_REQUIRE(a.rot_dims >= 0 && a.rot_dims % 2 == 0 && a.rot_dims <= a.dim, "layer %d: rotary dims %d of %d", i, a.rot_dims,
+                        a.dim);
+            QIE_REQUIRE(a.rot_layout == QIE_ROT_HALVES || a.rot_layout == QIE_ROT_INTERLEAVED, "layer %d: rotary layout %d", i,
+                        a.rot_layout);
+            QIE_REQUIRE((a.rot_dims == 0 && !a.rot_values) || a.rot_base > 0.f, "layer %d: rotary base", i);
+            QIE_REQUIRE(!a.rot_values || a.vdim % 2 == 0, "layer %d: turned values need an even vdim", i);
+            QIE_REQUIRE(a.mask >= QIE_MASK_CAUSAL && a.mask <= QIE_MASK_CHUNK && (a.mask == QIE_MASK_CAUSAL || a.mask_size > 0),
+                        "layer %d: mask %d of size %d", i, a.mask, a.mask_size);
+            QIE_REQUIRE(!a.values_are_keys || (a.vdim == a.dim && !a.rot_values), "layer %d: keys as values need vdim == dim", i);
+            if (d.mixer == QIE_MIXER_GQA_RECURRENT)
+                QIE_REQUIRE(d.rec.heads > 0 && d.rec.dim > 0 && d.rec.dim <= 512 && d.rec.vdim > 0, "layer %d: recurrence sizes", i);
+            continue;
+        }
         QIE_REQUIRE(d.mixer == QIE_MIXER_LATENT_ATTENTION, "layer %d: unknown mixer %d", i, d.mixer);
+        QIE_REQUIRE(arch->block == QIE_BLOCK_POSTNORM_GAIN, "layer %d: latent attention is wired to the post-norm block", i);
         QIE_REQUIRE(d.heads > 0 && d.dim > 0 && d.rot_dim >= 0 && d.vdim > 0 && d.kv_rank > 0 && d.window > 0,
                     "layer %d: invalid mixer sizes", i);
         QIE_REQUIRE(d.rot_dims >= 0 && d.rot_dims % 2 == 0 && d.rot_dims <= d.rot_dim, "layer %d: rotary dims %d of %d", i,
@@ -899,10 +1260,6 @@ int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* 
                         "layer %d: the layer it reads its cache from (%d) must own one of the same shape and rotation", i,
                         d.kv_from);
         }
-        QIE_REQUIRE(d.ff_kind >= QIE_FF_NONE && d.ff_kind <= QIE_FF_MOE, "layer %d: unknown feed-forward %d", i, d.ff_kind);
-        QIE_REQUIRE(d.ff_kind == QIE_FF_NONE || d.ff > 0, "layer %d: feed-forward size", i);
-        QIE_REQUIRE(d.ff_kind != QIE_FF_MOE || (d.experts > 0 && d.top > 0 && d.top <= d.experts), "layer %d: %d of %d experts", i,
-                    d.top, d.experts);
     }
     qie_engine* e = new qie_engine();
     if (opts) e->opts = *opts;
@@ -920,6 +1277,16 @@ int qie_engine_create_layered(const qie_arch_desc* arch, const qie_engine_opts* 
     for (int i = 0; i < arch->n_layers; i++) {
         m->L[i].d = m->descs[i];
         m->L[i].cache_layer = m->descs[i].kv_from >= 0 ? m->descs[i].kv_from : i;
+    }
+    m->loops = loops;
+    for (int i = 0; i < arch->n_layers; i++) {
+        if (loops && i == arch->loop_start) {
+            for (int t = 0; t < arch->loop_times; t++)
+                for (int j = arch->loop_start; j < arch->loop_stop; j++) m->runs.push_back(LayerRun{j, t > 0 && j == arch->loop_start});
+            i = arch->loop_stop - 1;
+            continue;
+        }
+        m->runs.push_back(LayerRun{i, false});
     }
     // informational mirror for qie_engine_spec
     e->spec.n_layers = arch->n_layers;
@@ -958,13 +1325,21 @@ int qie_engine_finalize_weights(qie_engine* e) {
     QIE_HIP(hipSetDevice(e->opts.device));
     const int64_t W = m->a.width, V = m->a.vocab;
     LM_GET(te, "embed", V, W);
-    LM_GET(th, "head", V, W);
-    LM_GET(tn, "final.norm");
     QIE_TRY(lm_alloc(m, &m->embed, (size_t)V * W * m->esz()));
     QIE_TRY(lm_upload_rows(m, m->embed, 0, W, *te));
-    QIE_TRY(lm_alloc(m, &m->head, (size_t)V * W * m->esz()));
-    QIE_TRY(lm_upload_rows(m, m->head, 0, W, *th));
-    m->g_final = host_elem(*tn, 0);
+    if (m->a.tied_head) {
+        m->head = m->embed;
+    } else {
+        LM_GET(th, "head", V, W);
+        QIE_TRY(lm_alloc(m, &m->head, (size_t)V * W * m->esz()));
+        QIE_TRY(lm_upload_rows(m, m->head, 0, W, *th));
+    }
+    if (m->a.block == QIE_BLOCK_SANDWICH) {
+        QIE_TRY(lm_vector(m, &m->w_final, "final.norm", W));
+    } else {
+        LM_GET(tn, "final.norm");
+        m->g_final = host_elem(*tn, 0);
+    }
     for (int i = 0; i < m->a.n_layers; i++) QIE_TRY(finalize_layer(e, m, i));
     m->host.clear();
     m->final = true;
@@ -1019,6 +1394,34 @@ int qie_batch_step(qie_batch* b, int32_t n_entries, const int32_t* slots, const 
     }
     QIE_TRY(flush_table(b));
     hipStream_t st = e->stream;
+    {   // the entries themselves (recurrent mixers walk an entry's rows in order) and their 16-row groups
+        s->h_ent.clear();
+        s->h_qgroups.clear();
+        int row = 0;
+        for (int i = 0; i < n_entries; i++) {
+            const int p0 = b->h_pos[slots[i]] - counts[i];
+            s->h_ent.push_back(int4{row, counts[i], slots[i], p0});
+            for (int k = 0; k < counts[i]; k += 16) s->h_qgroups.push_back(int4{row + k, std::min(16, counts[i] - k), slots[i], p0 + k});
+            row += counts[i];
+        }
+        if (n_entries > s->ent_cap || (int64_t)s->h_qgroups.size() > s->qgroups_cap) {
+            QIE_HIP(hipStreamSynchronize(st));
+            drop_graphs(s);
+            if (s->d_ent) hipFree(s->d_ent);
+            if (s->d_qgroups) hipFree(s->d_qgroups);
+            s->d_ent = s->d_qgroups = nullptr;
+            s->ent_cap = s->qgroups_cap = 0;
+            const int64_t ce = std::max<int64_t>(b->B, n_entries), cg = ((int64_t)s->h_qgroups.size() + 255) / 256 * 256;
+            QIE_TRY(dmalloc((void**)&s->d_ent, (size_t)ce * sizeof(int4)));
+            QIE_TRY(dmalloc((void**)&s->d_qgroups, (size_t)cg * sizeof(int4)));
+            s->ent_cap = ce;
+            s->qgroups_cap = cg;
+        }
+        QIE_HIP(hipMemcpyAsync(s->d_ent, s->h_ent.data(), s->h_ent.size() * sizeof(int4), hipMemcpyHostToDevice, st));
+        QIE_HIP(hipMemcpyAsync(s->d_qgroups, s->h_qgroups.data(), s->h_qgroups.size() * sizeof(int4), hipMemcpyHostToDevice, st));
+        s->n_ent = n_entries;
+        s->n_qgroups = (int)s->h_qgroups.size();
+    }
     QIE_HIP(hipMemcpyAsync(s->row_slot, hs, (size_t)T * 4, hipMemcpyHostToDevice, st));
     QIE_HIP(hipMemcpyAsync(s->row_pos, hs + R, (size_t)T * 4, hipMemcpyHostToDevice, st));
     QIE_HIP(hipMemcpyAsync(s->tok, hs + 2 * R, (size_t)T * 4, hipMemcpyHostToDevice, st));
@@ -1067,6 +1470,8 @@ int qie_batch_step_graphs(qie_batch* b, int32_t* n_graphs, int64_t* n_replays) {
     return 0;
 }
 
+int qie_engine_layer_runs(const qie_engine* e) { return e && e->lm ? (int)e->lm->runs.size() : 0; }
+
 int qie_batch_keep_layers(qie_batch* b, int32_t enable) {
     QIE_REQUIRE(b && b->lb, "qie_batch_keep_layers: a batch of a layered engine");
     b->lb->keep_on = enable != 0;
@@ -1077,7 +1482,7 @@ int qie_batch_step_layers(qie_batch* b, float* host_out, int64_t n) {
     QIE_REQUIRE(b && b->lb && host_out, "qie_batch_step_layers: bad arguments");
     LayeredBatch* s = b->lb;
     const LayeredModel* m = b->e->lm;
-    const int64_t W = m->a.width, T = s->last_T, L = m->a.n_layers;
+    const int64_t W = m->a.width, T = s->last_T, L = (int64_t)m->runs.size();
     QIE_REQUIRE(s->keep && T > 0 && n >= L * T * W, "qie_batch_step_layers: nothing kept, or the buffer is too small");
     QIE_HIP(hipStreamSynchronize(b->e->stream));
     for (int64_t i = 0; i < L; i++)
@@ -1086,7 +1491,7 @@ int qie_batch_step_layers(qie_batch* b, float* host_out, int64_t n) {
 }
 
 int qie_batch_time_stage(qie_batch* b, int32_t which, int32_t layer, int32_t iters, double* avg_us) {
-    QIE_REQUIRE(b && b->lb && avg_us && iters > 0 && which >= 0 && which <= 3, "qie_batch_time_stage: bad arguments");
+    QIE_REQUIRE(b && b->lb && avg_us && iters > 0 && which >= 0 && which <= 4, "qie_batch_time_stage: bad arguments");
     LayeredBatch* s = b->lb;
     const LayeredModel* m = b->e->lm;
     const int T = s->last_T;
@@ -1098,8 +1503,23 @@ int qie_batch_time_stage(qie_batch* b, int32_t which, int32_t layer, int32_t ite
     QIE_HIP(hipEventCreate(&e0));
     QIE_HIP(hipEventCreate(&e1));
     int rc = 0;
+    const bool gqa = which != 0 && m->L[layer].d.mixer != QIE_MIXER_LATENT_ATTENTION;
+    QIE_REQUIRE(which != 4 || m->L[layer].d.mixer == QIE_MIXER_GQA_RECURRENT, "qie_batch_time_stage: layer %d has no recurrence", layer);
+    int run = 0;   // the layer's first run
+    while (which != 0 && m->runs[run].layer != layer) run++;
     auto once = [&]() -> int {
         const float* xin = layer == 0 || which == 0 ? s->stack : s->x;
+        if (gqa) {   // the recurrence is timed from a zero state over the step's rows, the slots' states are not kept
+            const LayerDev& L = m->L[layer];
+            switch (which) {
+                case 1: return enq_gqa_attention(b, run, T);
+                case 2:
+                    QIE_TRY(enq_gqa_proj(b, run, T));
+                    return dense(b, s->ov, L.n_cat, L.wo, s->mix, m->a.width, T, m->a.width, L.n_cat, s->ov_bf);
+                case 3: return enq_ff(b, layer, T);
+                default: return enq_recurrence(b, run, T);
+            }
+        }
         switch (which) {
             case 0: return enq_forward(b, T, s->last_want);
             case 1: return enq_attention(b, layer, T);

@@ -11,8 +11,9 @@
 //   lay::head_gate         per-head sigmoid output gate
 //   lay::postnorm_add      y = x + g * v / sqrt(mean(v^2) + eps): a branch's result is normed, then added
 //   lay::depth_mix         x = sum_j a[j] X_j over the stack of earlier layer results
-//   lay::route_sigmoid_topk, moe_group, moe_gather, moe_combine: sigmoid router whose score
-//                          scales the expert's input, rows grouped by expert for the grouped linear
+//   lay::route_topk, moe_group, moe_gather, moe_combine: sigmoid router whose score scales the
+//                          expert's input, or biased logits whose softmax over the chosen ones
+//                          weights the outputs; rows grouped by expert for the grouped linear
 //   lay::silu_mul, embed_rows, final_rows, rows_to_bf16
 //
 // Everything the residual stream, a norm, a router, a score or a softmax touches is fp32.  No
@@ -490,7 +491,7 @@ int postnorm_add(const float* x, const float* v, float* y, uint16_t* y_bf, int T
 
 // rows picked by index, normed with one gain: out[i] = gain * x[rows[i]] / rms
 __global__ __launch_bounds__(256) void final_rows_kernel(const float* x, const int32_t* rows, float* out, uint16_t* out_bf, int W,
-                                                         float gain, float eps) {
+                                                         float gain, const float* w1p, float eps) {
     __shared__ float red[4];
     const int64_t t = rows[blockIdx.x];
     float ss = 0.f;
@@ -501,14 +502,14 @@ __global__ __launch_bounds__(256) void final_rows_kernel(const float* x, const i
     ss = block_sum256(ss, red);
     const float inv = gain / sqrtf(ss / (float)W + eps);
     for (int i = threadIdx.x; i < W; i += 256) {
-        const float o = x[t * W + i] * inv;
+        const float o = x[t * W + i] * inv * (w1p ? 1.0f + w1p[i] : 1.0f);
         out[(int64_t)blockIdx.x * W + i] = o;
         if (out_bf) out_bf[(int64_t)blockIdx.x * W + i] = f2bf(o);
     }
 }
-int final_rows(const float* x, const int32_t* rows, float* out, uint16_t* out_bf, int n, int W, float gain, float eps,
-               hipStream_t st) {
-    hipLaunchKernelGGL(final_rows_kernel, dim3(n), dim3(256), 0, st, x, rows, out, out_bf, W, gain, eps);
+int final_rows(const float* x, const int32_t* rows, float* out, uint16_t* out_bf, int n, int W, float gain, const float* w1p,
+               float eps, hipStream_t st) {
+    hipLaunchKernelGGL(final_rows_kernel, dim3(n), dim3(256), 0, st, x, rows, out, out_bf, W, gain, w1p, eps);
     QIE_LAUNCH_CHECK();
     return 0;
 }
@@ -556,8 +557,8 @@ int silu_mul(const float* gu, float* a, uint16_t* a_bf, int64_t M, int ff, hipSt
 // descending order -> sel[t, k], score[t, k].  The ranking compares z, which orders the experts
 // as s does but does not saturate (sigmoid(z) is 1.0f for every z above ~17).  One block per row.
 template <typename TW>
-__global__ __launch_bounds__(256) void route_kernel(const float* y, const TW* Wr, int W, int E, int top, int32_t* sel,
-                                                    float* score) {
+__global__ __launch_bounds__(256) void route_kernel(const float* y, const TW* Wr, const float* bias, int W, int E, int top, int mode,
+                                                    int32_t* sel, float* score) {
     extern __shared__ float s[];   // [E] router logits
     const int64_t t = blockIdx.x;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -565,10 +566,11 @@ __global__ __launch_bounds__(256) void route_kernel(const float* y, const TW* Wr
         float z = 0.f;
         for (int i = lane; i < W; i += 64) z = fmaf(y[t * W + i], ldf<TW>(Wr, (int64_t)e * W + i), z);
         z = wave_sum(z);
-        if (lane == 0) s[e] = z;
+        if (lane == 0) s[e] = bias ? z + bias[e] : z;
     }
     __syncthreads();
     if (threadIdx.x == 0) {
+        float z0 = 0.f, den = 0.f;
         for (int k = 0; k < top; k++) {
             int best = -1;
             float bv = 0.f;
@@ -579,19 +581,29 @@ __global__ __launch_bounds__(256) void route_kernel(const float* y, const TW* Wr
                 }
             if (best < 0) best = 0;   // only if logits are not finite
             sel[t * top + k] = best;
-            score[t * top + k] = 1.0f / (1.0f + expf(-bv));
+            if (mode == 0) {
+                score[t * top + k] = 1.0f / (1.0f + expf(-bv));
+            } else {   // softmax over the chosen logits: the first chosen is the largest
+                if (k == 0) z0 = bv;
+                const float ex = expf(bv - z0);
+                score[t * top + k] = ex;
+                den += ex;
+            }
             s[best] = -INFINITY;
         }
+        if (mode != 0)
+            for (int k = 0; k < top; k++) score[t * top + k] /= den;
     }
 }
-int route_sigmoid_topk(const float* y, const void* Wr, bool w_f32, int T, int W, int E, int top, int32_t* sel, float* score,
-                       hipStream_t st) {
+int route_topk(const float* y, const void* Wr, const float* bias, bool w_f32, int T, int W, int E, int top, int mode, int32_t* sel,
+               float* score, hipStream_t st) {
     QIE_REQUIRE(top >= 1 && top <= E && E <= 8192, "router: top %d of %d experts", top, E);
     if (w_f32)
-        hipLaunchKernelGGL(route_kernel<float>, dim3(T), dim3(256), (size_t)E * 4, st, y, (const float*)Wr, W, E, top, sel, score);
+        hipLaunchKernelGGL(route_kernel<float>, dim3(T), dim3(256), (size_t)E * 4, st, y, (const float*)Wr, bias, W, E, top, mode,
+                           sel, score);
     else
-        hipLaunchKernelGGL(route_kernel<uint16_t>, dim3(T), dim3(256), (size_t)E * 4, st, y, (const uint16_t*)Wr, W, E, top, sel,
-                           score);
+        hipLaunchKernelGGL(route_kernel<uint16_t>, dim3(T), dim3(256), (size_t)E * 4, st, y, (const uint16_t*)Wr, bias, W, E, top,
+                           mode, sel, score);
     QIE_LAUNCH_CHECK();
     return 0;
 }
@@ -648,7 +660,7 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(const float* y, const f
                                                          float* xg, uint16_t* xg_bf) {
     const int64_t i = blockIdx.x;
     const int64_t t = i / top, d = slot_of[i];
-    const float s = score[i];
+    const float s = score ? score[i] : 1.0f;
     for (int w = threadIdx.x; w < W; w += 256) {
         const float o = s * y[t * W + w];
         xg[d * W + w] = o;
@@ -661,17 +673,21 @@ int moe_gather(const float* y, const float* score, const int32_t* slot_of, int T
     QIE_LAUNCH_CHECK();
     return 0;
 }
-// f[t, :] = sum_k yd[slot_of[t * top + k], :]
-__global__ __launch_bounds__(256) void moe_combine_kernel(const float* yd, const int32_t* slot_of, int top, int W, float* f) {
+// f[t, :] = sum_k (score[t * top + k] or 1) * yd[slot_of[t * top + k], :]
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* yd, const int32_t* slot_of, const float* score, int top, int W,
+                                                          float* f) {
     const int64_t t = blockIdx.x;
     for (int w = threadIdx.x; w < W; w += 256) {
         float s = 0.f;
-        for (int k = 0; k < top; k++) s += yd[(int64_t)slot_of[t * top + k] * W + w];
+        if (score)
+            for (int k = 0; k < top; k++) s = fmaf(score[t * top + k], yd[(int64_t)slot_of[t * top + k] * W + w], s);
+        else
+            for (int k = 0; k < top; k++) s += yd[(int64_t)slot_of[t * top + k] * W + w];
         f[t * W + w] = s;
     }
 }
-int moe_combine(const float* yd, const int32_t* slot_of, int T, int top, int W, float* f, hipStream_t st) {
-    hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, st, yd, slot_of, top, W, f);
+int moe_combine(const float* yd, const int32_t* slot_of, const float* score, int T, int top, int W, float* f, hipStream_t st) {
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, st, yd, slot_of, score, top, W, f);
     QIE_LAUNCH_CHECK();
     return 0;
 }

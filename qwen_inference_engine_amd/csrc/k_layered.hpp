@@ -96,6 +96,104 @@ constexpr int kLatentQG = 1;   // 2 measured slower at kv_rank 256 (one wave per
 bool latent_attention_mfma_fits(int R, int rot);
 int latent_attention_mfma(const LatentAttnMfmaP& p, hipStream_t st);
 
+// ------------------------------------------------------------------ grouped-query attention
+// (k_mixers.hip)  Paged K / V rows: inside a page the K rows of one cache region start at k_off
+// and are kv_heads * dim wide, its V rows at v_off, kv_heads * vdim wide (LatentCache names the
+// pool, its block table and the page geometry).
+//
+// gqa_post: per row of the fused projection, every query and key head is RMS-normed over dim
+// (qk_norm: 0 no, 1 with the weight qn_w / kn_w, 2 without one), its first rot_dims coordinates
+// are turned by the row's position (layout 0: i with i + rot_dims / 2; 1: 2i with 2i + 1); queries
+// go back in place, keys to the cache.  Values: v_col < 0 caches the key as projected (before its
+// norm) as the value; else W_v's columns, turned over all vdim coordinates when rot_values.
+struct GqaPostP {
+    float* proj;
+    int64_t ld;
+    int q_col, k_col, v_col;
+    const int32_t* row_slot;
+    const int32_t* row_pos;
+    int heads, kv_heads, dim, vdim;
+    int qk_norm;
+    const float* qn_w;
+    const float* kn_w;
+    float eps;
+    int rot_dims, rot_layout;
+    const float* rope_cos;    // [positions][rot_dims / 2]
+    const float* rope_sin;
+    int rot_values;
+    const float* vrope_cos;   // [positions][vdim / 2]
+    const float* vrope_sin;
+    LatentCache cache;
+    int64_t k_off, v_off;
+};
+int gqa_post(const GqaPostP& p, bool cache_f32, int T, hipStream_t st);
+
+// Softmax attention of every (row, head) over the keys its mask lets it see (mask 0: all j <= i;
+// 1: the last mask_size; 2: those with j / mask_size == i / mask_size); score = q.k * scale
+// - r1[h] * ln(1 + r2[h] * (i - j)) when r1 is set.  rot_values: the weighted sum is turned back
+// by the row's position.  The result times out_scale goes to out[t * ld_out + out_col + h * vdim
+// ...] (and its bf16 image).
+struct GqaAttnP {
+    const float* proj;
+    int64_t ld;
+    int q_col;
+    const int32_t* row_slot;
+    const int32_t* row_pos;
+    int heads, kv_heads, dim, vdim;
+    int mask, mask_size;
+    float scale;
+    const float* r1;
+    const float* r2;
+    int rot_values, rot_layout;
+    const float* vrope_cos;
+    const float* vrope_sin;
+    LatentCache cache;
+    int64_t k_off, v_off;
+    float out_scale;
+    float* out;
+    uint16_t* out_bf;
+    int64_t ld_out;
+    int out_col;
+};
+int gqa_attention(const GqaAttnP& p, bool cache_f32, int T, hipStream_t st);
+// The matrix-core form for bf16 caches (dim and vdim multiples of 32 up to 256): one wave per 16
+// consecutive rows of one entry and head.  groups: {first packed row, rows, slot, first position}.
+struct GqaAttnMfmaP {
+    GqaAttnP a;
+    const int4* groups;
+    int n_groups;
+};
+bool gqa_attention_mfma_fits(int dim, int vdim);
+int gqa_attention_mfma(const GqaAttnMfmaP& p, hipStream_t st);
+
+// ------------------------------------------------------------------ gated linear recurrence
+// Per entry {first packed row, rows, slot, first position} and head: S [dim][vdim] (fp32, at
+// state + slot * slot_stride + state_off) runs through the entry's rows in order,
+// S = diag(f) S + (1 - f) v^T, o = S^T q, with q = silu(proj[q_col ...]),
+// f = lower + (1 - lower) * sigmoid(proj[f_col ...] + f_bias); an entry whose first position is 0
+// starts from S = 0.  Raw o -> out [T][heads * vdim].
+struct GatedScanP {
+    const float* proj;
+    int64_t ld;
+    int q_col, f_col, v_col;
+    const int4* entries;
+    int n_entries;
+    int heads, dim, vdim;
+    const float* f_bias;
+    const float* lower;
+    float* state;
+    int64_t slot_stride, state_off;
+    float* out;
+};
+int gated_scan(const GatedScanP& p, hipStream_t st);
+// out[t, out_col + h * vdim + c] = scale * o[t, h, c] / sqrt(mean_c o^2 + eps) * w[c]
+int head_norm_rows(const float* o, const float* w, float eps, float scale, int heads, int vdim, int T, float* out, uint16_t* out_bf,
+                   int64_t ld_out, int out_col, hipStream_t st);
+// Rows of W: x = xin + rms(v) * (1 + wb) (when v) + add (when add); then (when wn)
+// h = rms(x) * (1 + wn) with its bf16 image.  xin may be x.
+int add_norm(float* x, const float* xin, const float* v, const float* wb, const float* add, const float* wn, float* h, uint16_t* h_bf,
+             int T, int W, float eps, hipStream_t st);
+
 // The producers below also write the bf16 image of their result when the *_bf pointer is set
 // (bf16 engines: the next product reads it; no separate rounding pass).
 int embed_rows(const void* E, bool w_f32, const int32_t* tok, float* out, uint16_t* out_bf, int T, int W, int vocab,
@@ -103,16 +201,20 @@ int embed_rows(const void* E, bool w_f32, const int32_t* tok, float* out, uint16
 int head_gate(float* v, uint16_t* v_bf, const float* proj, int64_t ld, int g_col, int heads, int vd, int T, hipStream_t st);
 // y = (x ? x : 0) + gain * v / sqrt(mean(v^2) + eps), rows of W
 int postnorm_add(const float* x, const float* v, float* y, uint16_t* y_bf, int T, int W, float gain, float eps, hipStream_t st);
-int final_rows(const float* x, const int32_t* rows, float* out, uint16_t* out_bf, int n, int W, float gain, float eps,
-               hipStream_t st);
+// out[i] = gain * rms(x[rows[i]]) (* (1 + w1p) when w1p)
+int final_rows(const float* x, const int32_t* rows, float* out, uint16_t* out_bf, int n, int W, float gain, const float* w1p,
+               float eps, hipStream_t st);
 int depth_mix(const float* stack, int64_t stride, const float* a, int n, float* x, uint16_t* x_bf, int64_t count, hipStream_t st);
 int silu_mul(const float* gu, float* a, uint16_t* a_bf, int64_t M, int ff, hipStream_t st);
-int route_sigmoid_topk(const float* y, const void* Wr, bool w_f32, int T, int W, int E, int top, int32_t* sel, float* score,
-                       hipStream_t st);
+// mode 0: score = sigmoid(z) of the `top` largest z = W_r y; mode 1: z = W_r y + bias, score = the
+// softmax over the `top` largest z alone.  Ties: the lower index.
+int route_topk(const float* y, const void* Wr, const float* bias, bool w_f32, int T, int W, int E, int top, int mode, int32_t* sel,
+               float* score, hipStream_t st);
 int moe_group(const int32_t* sel, int n, int E, int32_t* cnt, int32_t* off, int32_t* slot_of, hipStream_t st);
+// score (may be null: 1) scales the gathered input rows / the combined output rows
 int moe_gather(const float* y, const float* score, const int32_t* slot_of, int T, int top, int W, float* xg, uint16_t* xg_bf,
                hipStream_t st);
-int moe_combine(const float* yd, const int32_t* slot_of, int T, int top, int W, float* f, hipStream_t st);
+int moe_combine(const float* yd, const int32_t* slot_of, const float* score, int T, int top, int W, float* f, hipStream_t st);
 int argmax_rows(const float* x, int M, int64_t V, int32_t* ids, hipStream_t st);
 int rows_to_bf16(const float* x, uint16_t* y, int64_t n, hipStream_t st);
 int rows_to_bf16_strided(const float* x, int64_t ldx, uint16_t* y, int64_t ldy, int64_t M, int K, hipStream_t st);

@@ -327,9 +327,9 @@ class Batch:
         _lib.check(self.lib.qie_batch_keep_layers(self.h, int(on)), "qie_batch_keep_layers")
 
     def step_layers(self, rows: int) -> np.ndarray:
-        """The residual stream after every layer of the last step, float32 [layers, rows, width]
-        (after keep_layers())."""
-        out = np.zeros((self.e.spec.n_layers, rows, self.e.spec.width), dtype=np.float32)
+        """The residual stream after every layer run of the last step (a repeated layer counts each
+        time), float32 [layer runs, rows, width] (after keep_layers())."""
+        out = np.zeros((self.e.spec.n_runs, rows, self.e.spec.width), dtype=np.float32)
         _lib.check(self.lib.qie_batch_step_layers(self.h, out.ctypes.data_as(C.POINTER(C.c_float)), out.size),
                    "qie_batch_step_layers")
         return out

@@ -185,16 +185,57 @@ class LatentAttention:
 
 
 @dataclasses.dataclass(frozen=True)
+class GqaAttention:
+    """Mixer: grouped-query softmax attention over a paged K / V cache; every option is a field
+    (qie_gqa_desc): head norms, rotary pairing and extent, turned values, mask, keys as values,
+    log-distance bias."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    qk_norm: str = "none"        # "none" | "weight" | "plain"
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    rot_layout: str = "halves"   # "halves" (i, i + dims/2) | "interleaved" (2i, 2i + 1)
+    rot_values: bool = False
+    mask: str = "causal"         # "causal" | "window" | "chunk"
+    mask_size: int = 0
+    values_are_keys: bool = False
+    dist_bias: bool = False
+
+
+@dataclasses.dataclass(frozen=True)
+class GatedRecurrence:
+    """Gated linear recurrence (HGRN2 form): a [dim, vdim] fp32 state per head and slot."""
+    heads: int
+    dim: int
+    vdim: int
+
+
+@dataclasses.dataclass(frozen=True)
+class AttentionWithRecurrence:
+    """Mixer: a GqaAttention and a GatedRecurrence read the same input; their results are added
+    with fixed scales."""
+    attn: GqaAttention
+    rec: GatedRecurrence
+    attn_scale: float
+    rec_scale: float
+
+
+@dataclasses.dataclass(frozen=True)
 class FeedForward:
     kind: str         # "dense" or "moe"
     ff: int           # hidden size (of one expert for "moe")
     experts: int = 0
     top: int = 0
+    router: str = "sigmoid_in"   # "sigmoid_in": sigmoid scores scale the input; "softmax_out":
+                                 # biased logits, softmax over the chosen ones weights the output
 
 
 @dataclasses.dataclass(frozen=True)
 class LayerSpec:
-    mixer: LatentAttention
+    mixer: object     # LatentAttention | GqaAttention | AttentionWithRecurrence
     mlp: Optional[FeedForward]
 
 
@@ -206,10 +247,25 @@ class LayeredSpec:
     norm_eps: float
     layers: Tuple[LayerSpec, ...]
     depth_mix: bool = True
+    block: str = "postnorm_gain"     # "postnorm_gain" | "sandwich" (weight-vector norms around every branch)
+    tied_head: bool = False
+    loop: Optional[Tuple[int, int, int]] = None   # (start, stop, times): layers [start, stop) run `times` times
 
     @property
     def n_layers(self) -> int:
         return len(self.layers)
+
+    def runs(self) -> List[int]:
+        """Layer index of every layer run, in execution order."""
+        n = len(self.layers)
+        if not self.loop or self.loop[2] <= 1 or self.loop[1] <= self.loop[0]:
+            return list(range(n))
+        a, b, t = self.loop
+        return list(range(a)) + list(range(a, b)) * t + list(range(b, n))
+
+    @property
+    def n_runs(self) -> int:
+        return len(self.runs())
 
     @property
     def hidden(self) -> int:
@@ -218,40 +274,89 @@ class LayeredSpec:
     def to_c(self):
         """(ArchDescC, keepalive of its layer array)."""
         arr = (_lib.LayerDescC * len(self.layers))()
+        def gqa(g, m):
+            g.heads, g.kv_heads, g.dim, g.vdim, g.scale = m.heads, m.kv_heads, m.dim, m.vdim, m.scale
+            g.qk_norm = {"none": _lib.QIE_QKNORM_NONE, "weight": _lib.QIE_QKNORM_WEIGHT, "plain": _lib.QIE_QKNORM_PLAIN}[m.qk_norm]
+            g.rot_dims, g.rot_base = m.rot_dims, m.rot_base
+            g.rot_layout = {"halves": _lib.QIE_ROT_HALVES, "interleaved": _lib.QIE_ROT_INTERLEAVED}[m.rot_layout]
+            g.rot_values = int(m.rot_values)
+            g.mask = {"causal": _lib.QIE_MASK_CAUSAL, "window": _lib.QIE_MASK_WINDOW, "chunk": _lib.QIE_MASK_CHUNK}[m.mask]
+            g.mask_size, g.values_are_keys, g.dist_bias = m.mask_size, int(m.values_are_keys), int(m.dist_bias)
+
         for d, L in zip(arr, self.layers):
             m = L.mixer
-            d.mixer = _lib.QIE_MIXER_LATENT_ATTENTION
-            d.heads, d.dim, d.rot_dim, d.vdim, d.kv_rank = m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank
-            d.window, d.kv_from, d.rot_dims = m.window, -1 if m.kv_from is None else m.kv_from, m.rot_dims
-            d.rot_base, d.scale = m.rot_base, m.scale
+            if isinstance(m, GqaAttention):
+                d.mixer = _lib.QIE_MIXER_GQA
+                gqa(d.gqa, m)
+            elif isinstance(m, AttentionWithRecurrence):
+                d.mixer = _lib.QIE_MIXER_GQA_RECURRENT
+                gqa(d.gqa, m.attn)
+                d.rec.heads, d.rec.dim, d.rec.vdim = m.rec.heads, m.rec.dim, m.rec.vdim
+                d.gqa_scale, d.rec_scale = m.attn_scale, m.rec_scale
+            else:
+                d.mixer = _lib.QIE_MIXER_LATENT_ATTENTION
+                d.heads, d.dim, d.rot_dim, d.vdim, d.kv_rank = m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank
+                d.window, d.kv_from, d.rot_dims = m.window, -1 if m.kv_from is None else m.kv_from, m.rot_dims
+                d.rot_base, d.scale = m.rot_base, m.scale
             if L.mlp is None:
                 d.ff_kind = _lib.QIE_FF_NONE
             elif L.mlp.kind == "dense":
                 d.ff_kind, d.ff = _lib.QIE_FF_DENSE, L.mlp.ff
             else:
                 d.ff_kind, d.ff, d.experts, d.top = _lib.QIE_FF_MOE, L.mlp.ff, L.mlp.experts, L.mlp.top
+                d.router = _lib.QIE_ROUTER_SOFTMAX_OUT if L.mlp.router == "softmax_out" else _lib.QIE_ROUTER_SIGMOID_IN
         a = _lib.ArchDescC()
         a.n_layers, a.width, a.vocab, a.norm_eps = len(self.layers), self.width, self.vocab, self.norm_eps
         a.depth_mix = int(self.depth_mix)
+        a.block = _lib.QIE_BLOCK_SANDWICH if self.block == "sandwich" else _lib.QIE_BLOCK_POSTNORM_GAIN
+        a.tied_head = int(self.tied_head)
+        if self.loop:
+            a.loop_start, a.loop_stop, a.loop_times = self.loop
         a.layers = arr
         return a, arr
 
     def tensor_shapes(self) -> "dict[str, List[int]]":
         """Checkpoint tensor names and shapes of this architecture."""
         W, out = self.width, {"embed": [self.vocab, self.width]}
+        sandwich = self.block == "sandwich"
+        nshape = [W] if sandwich else []
+
+        def gqa(q, m):
+            out[q + "q"], out[q + "k"] = [m.heads * m.dim, W], [m.kv_heads * m.dim, W]
+            if not m.values_are_keys:
+                out[q + "v"] = [m.kv_heads * m.vdim, W]
+            if m.qk_norm == "weight":
+                out[q + "q.norm"], out[q + "k.norm"] = [m.dim], [m.dim]
+            if m.dist_bias:
+                out[q + "r1"], out[q + "r2"] = [m.heads], [m.heads]
+            out[q + "o"] = [W, m.heads * m.vdim]
+
         for i, L in enumerate(self.layers):
             m, p = L.mixer, f"l{i}."
-            out[p + "norm1"] = []
+            out[p + "norm1"] = nshape
+            if sandwich:
+                out[p + "norm1b"] = nshape
             if L.mlp is not None:
-                out[p + "norm2"] = []
-            out[p + "mix.q"] = [m.heads * (m.dim + m.rot_dim), W]
-            if m.kv_from is None:
-                out[p + "mix.dkv"] = [m.kv_rank + m.rot_dim, W]
-                out[p + "mix.dkv.norm"] = [m.kv_rank]
-            out[p + "mix.uk"] = [m.heads * m.dim, m.kv_rank]
-            out[p + "mix.uv"] = [m.heads * m.vdim, m.kv_rank]
-            out[p + "mix.g"] = [m.heads, W]
-            out[p + "mix.o"] = [W, m.heads * m.vdim]
+                out[p + "norm2"] = nshape
+                if sandwich:
+                    out[p + "norm2b"] = nshape
+            if isinstance(m, GqaAttention):
+                gqa(p + "mix.", m)
+            elif isinstance(m, AttentionWithRecurrence):
+                gqa(p + "mix.left.", m.attn)
+                r, c = p + "mix.right.", m.rec
+                out[r + "q"], out[r + "f"], out[r + "v"] = [c.heads * c.dim, W], [c.heads * c.dim, W], [c.heads * c.vdim, W]
+                out[r + "f.b"], out[r + "lower"], out[r + "norm"] = [c.heads * c.dim], [c.heads * c.dim], [c.vdim]
+                out[r + "o"] = [W, c.heads * c.vdim]
+            else:
+                out[p + "mix.q"] = [m.heads * (m.dim + m.rot_dim), W]
+                if m.kv_from is None:
+                    out[p + "mix.dkv"] = [m.kv_rank + m.rot_dim, W]
+                    out[p + "mix.dkv.norm"] = [m.kv_rank]
+                out[p + "mix.uk"] = [m.heads * m.dim, m.kv_rank]
+                out[p + "mix.uv"] = [m.heads * m.vdim, m.kv_rank]
+                out[p + "mix.g"] = [m.heads, W]
+                out[p + "mix.o"] = [W, m.heads * m.vdim]
             if L.mlp is not None and L.mlp.kind == "dense":
                 out.update({p + "mlp.gate": [L.mlp.ff, W], p + "mlp.up": [L.mlp.ff, W], p + "mlp.down": [W, L.mlp.ff]})
             elif L.mlp is not None:
@@ -259,21 +364,53 @@ class LayeredSpec:
                     q = f"{p}mlp.e{e}."
                     out.update({q + "gate": [L.mlp.ff, W], q + "up": [L.mlp.ff, W], q + "down": [W, L.mlp.ff]})
                 out[p + "mlp.router"] = [L.mlp.experts, W]
+                if L.mlp.router == "softmax_out":
+                    out[p + "mlp.router.b"] = [L.mlp.experts]
             if self.depth_mix:
                 out[p + "dwa"] = [i + 2]
-        out["final.norm"] = []
-        out["head"] = [self.vocab, W]
+        out["final.norm"] = nshape
+        if not self.tied_head:
+            out["head"] = [self.vocab, W]
         return out
 
     def cache_row_elems(self) -> int:
-        """Cached elements per token, all caching layers together."""
-        return sum(L.mixer.kv_rank + L.mixer.rot_dim for L in self.layers if L.mixer.kv_from is None)
+        """Cached elements per token, all layer runs together."""
+        n = 0
+        for i in self.runs():
+            m = self.layers[i].mixer
+            if isinstance(m, LatentAttention):
+                n += m.kv_rank + m.rot_dim if m.kv_from is None else 0
+            else:
+                a = m.attn if isinstance(m, AttentionWithRecurrence) else m
+                n += a.kv_heads * (a.dim + a.vdim)
+        return n
+
+    def state_elems(self) -> int:
+        """fp32 state elements per slot (recurrent mixers), all layer runs together."""
+        return sum(self.layers[i].mixer.rec.heads * self.layers[i].mixer.rec.dim * self.layers[i].mixer.rec.vdim
+                   for i in self.runs() if isinstance(self.layers[i].mixer, AttentionWithRecurrence))
 
     def step_flops(self, rows: int, ctx: int) -> float:
         """Multiply-adds x 2 of one step of `rows` tokens whose windows hold about `ctx` keys."""
         W, f = self.width, 0.0
-        for L in self.layers:
+        for i in self.runs():
+            L = self.layers[i]
             m = L.mixer
+            if not isinstance(m, LatentAttention):
+                a = m.attn if isinstance(m, AttentionWithRecurrence) else m
+                n_in = a.heads * a.dim + a.kv_heads * (a.dim + (0 if a.values_are_keys else a.vdim))
+                n_cat = a.heads * a.vdim
+                keys = ctx if a.mask == "causal" else min(ctx, a.mask_size if a.mask == "window" else (a.mask_size + 1) // 2)
+                f += 2.0 * rows * a.heads * keys * (a.dim + a.vdim)
+                if isinstance(m, AttentionWithRecurrence):
+                    c = m.rec
+                    n_in += c.heads * (2 * c.dim + c.vdim)
+                    n_cat += c.heads * c.vdim
+                    f += 2.0 * rows * c.heads * c.dim * c.vdim * 2
+                f += 2.0 * rows * W * (n_in + n_cat)
+                if L.mlp is not None:
+                    f += 2.0 * rows * (1 if L.mlp.kind == "dense" else L.mlp.top) * 3 * W * L.mlp.ff
+                continue
             n_in = m.heads * (m.dim + m.rot_dim) + m.heads + (m.kv_rank + m.rot_dim if m.kv_from is None else 0)
             f += 2.0 * rows * W * n_in + 2.0 * rows * m.heads * m.kv_rank * (m.dim + m.vdim) + 2.0 * rows * W * m.heads * m.vdim
             f += 2.0 * rows * m.heads * min(ctx, m.window) * (2 * m.kv_rank + m.rot_dim)
@@ -308,7 +445,44 @@ def _tivazen_from_config(cfg: dict, name: str) -> LayeredSpec:
     return LayeredSpec(name, int(cfg["width"]), int(cfg["vocab"]), float(cfg["norm"]["eps"]), tuple(layers), True)
 
 
-ARCHITECTURES = {"Tivazen": _tivazen_from_config}
+def _nodutar_from_config(cfg: dict, name: str) -> LayeredSpec:
+    """Nodutar: sandwich-normed blocks whose mixer is either a block-local grouped-query attention
+    (normed, partly rotated queries and keys, values turned by their position) beside a gated
+    linear recurrence, or a causal attention whose values are its keys and whose scores carry a
+    log-distance bias; softmax-routed experts; an optional repeated group of layers; tied head."""
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        m = L["mixer"]
+        if L["type"] == "parallel":
+            a, c = m["left"], m["right"]
+            attn = GqaAttention(
+                heads=int(a["heads"]), kv_heads=int(a["kv_heads"]), dim=int(a["dim"]), vdim=int(a["vdim"]), scale=float(a["scale"]),
+                qk_norm="weight", rot_dims=int(a["rot"]["dims"]), rot_base=float(a["rot"]["base"]), rot_layout="interleaved",
+                rot_values=True, mask="chunk", mask_size=int(a["mask"]["size"]))
+            rec = GatedRecurrence(heads=int(c["heads"]), dim=int(c["dim"]), vdim=int(c["vdim"]))
+            mixer = AttentionWithRecurrence(attn, rec, float(m["left_scale"]), float(m["right_scale"]))
+        elif L["type"] == "attention":
+            mixer = GqaAttention(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["dim"]),
+                                 scale=float(m["scale"]), qk_norm="plain", mask="causal", values_are_keys=True, dist_bias=True)
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {L['type']!r}")
+        f = L.get("mlp")
+        if f is None:
+            mlp = None
+        elif f["kind"] == "moe":
+            mlp = FeedForward("moe", int(f["expert"]["ff"]), int(f["router"]["experts"]), int(f["router"]["top"]), "softmax_out")
+        else:
+            raise ValueError(f"layer {i}: unknown feed-forward kind {f['kind']!r}")
+        layers.append(LayerSpec(mixer, mlp))
+    lp = cfg.get("loop")
+    loop = (int(lp["start"]), int(lp["stop"]), int(lp["times"])) if lp else None
+    if loop and not (0 <= loop[0] <= loop[1] <= len(layers) and loop[2] >= 1):
+        raise ValueError(f"loop {loop} does not fit {len(layers)} layers")
+    return LayeredSpec(name, int(cfg["width"]), int(cfg["vocab"]), float(cfg["norm"]["eps"]), tuple(layers), depth_mix=False,
+                       block="sandwich", tied_head=True, loop=loop)
+
+
+ARCHITECTURES = {"Tivazen": _tivazen_from_config, "Nodutar": _nodutar_from_config}
 
 
 def spec_from_config(cfg: dict, name: str = "model", numerics: str = "hf"):
