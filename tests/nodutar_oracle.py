@@ -131,7 +131,9 @@ def moe_ff(h, mlp, T, pfx):
     z = h @ T[pfx + "router"].T + T[pfx + "router.b"]
     out = np.zeros((h.shape[0], T[pfx + "e0.down"].shape[0]))
     for t in range(h.shape[0]):
-        idx = np.argsort(-z[t], kind="stable")[:top]
+        # ranked on logits rounded far below any real difference: rows of W_r that are equal give
+        # equal logits here, whatever order the matrix product summed them in
+        idx = np.argsort(-np.round(z[t], 10), kind="stable")[:top]
         w = softmax_rows(z[t, idx])
         for wt, e in zip(w, idx):
             p = f"{pfx}e{e}."
