@@ -56,6 +56,15 @@ LAYERED_SIZES = {
 }
 
 
+# Sizes of `--nodutar`: (width, heads, kv heads, head dim, rotary dims, block of the block-local mask,
+# recurrence heads, recurrence dim, recurrence vdim, experts, top, expert ff, vocab).  Four layers: attention
+# beside recurrence, distance-biased attention, attention beside recurrence, distance-biased attention; all routed.
+NODUTAR_SIZES = {
+    "1k": (1024, 16, 4, 64, 32, 512, 8, 64, 128, 8, 2, 704, 32000),
+    "2k": (2048, 16, 4, 128, 64, 1024, 16, 64, 128, 8, 2, 1408, 32000),
+}
+
+
 def parse(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -96,6 +105,10 @@ def parse(argv=None):
                     help="instead of the default workload: prefill and decode throughput of a layered (Tivazen) "
                          "model at this size with random weights, per-stage times, and the Qwen decoder at "
                          "equal width / heads / ffn / layers beside it (one JSON line of its own)")
+    ap.add_argument("--nodutar", choices=sorted(NODUTAR_SIZES), default=None,
+                    help="instead of the default workload: prefill and decode throughput of a Nodutar model at this "
+                         "size with random weights, per-stage times, and the Qwen decoder at equal width / heads / "
+                         "layers beside it (one JSON line of its own)")
     ap.add_argument("--dry-run", action="store_true",
                     help="launcher only: print the child ranks' environments as JSON and exit (no GPU)")
     return ap.parse_args(argv)
@@ -151,6 +164,8 @@ def main(argv=None):
         return 0
     if a.layered:
         return run_layered(a)
+    if a.nodutar:
+        return run_nodutar(a)
     return run(a)
 
 
@@ -177,6 +192,146 @@ def layered_model(S, size):
             v = (np.resize(np.roll(pool, 7919 * k), n) * fan ** -0.5).reshape(shape)
         tensors[name] = (np.ascontiguousarray(v, np.float32).view(np.uint32) >> 16).astype(np.uint16).reshape(shape)
     return spec, tensors
+
+
+def nodutar_model(S, size):
+    """(LayeredSpec, {name: bf16 words}) at one of NODUTAR_SIZES, random weights from one pool."""
+    W, H, G, hd, rot, blk, RH, rd, rv, E, top, eff, V = NODUTAR_SIZES[size]
+    moe = {"kind": "moe", "expert": {"ff": eff}, "router": {"experts": E, "top": top}}
+    par = {"type": "parallel", "mlp": moe, "mixer": {
+        "left": {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "mask": {"size": blk}, "rot": {"base": 10000.0, "dims": rot},
+                 "scale": hd ** -0.5},
+        "right": {"heads": RH, "dim": rd, "vdim": rv}, "left_scale": 0.8, "right_scale": 0.5}}
+    att = {"type": "attention", "mlp": moe, "mixer": {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5 * 4}}
+    cfg = {"architecture": "Nodutar", "layers": [par, att, par, att], "norm": {"eps": 1e-6}, "vocab": V, "width": W}
+    spec = S.spec_from_config(cfg, name=f"nodutar-{size}")
+    pool = np.random.default_rng(0).standard_normal(1 << 22).astype(np.float32)
+    tensors = {}
+    for k, (name, shape) in enumerate(spec.tensor_shapes().items()):
+        n = int(np.prod(shape))
+        if name.endswith(("q.norm", "k.norm", "right.norm")):
+            v = np.ones(shape, np.float32)
+        elif name.endswith(("norm1", "norm1b", "norm2", "norm2b", "final.norm", "router.b", "f.b")):
+            v = np.zeros(shape, np.float32)
+        elif name.endswith("lower"):
+            v = np.linspace(0.1, 0.95, n, dtype=np.float32).reshape(shape)
+        elif name.endswith(("r1", "r2")):
+            v = np.full(shape, 0.5, np.float32)
+        else:
+            fan = shape[-1] if name != "embed" else 1
+            v = (np.resize(np.roll(pool, 7919 * k), n) * fan ** -0.5).reshape(shape)
+        tensors[name] = (np.ascontiguousarray(v, np.float32).view(np.uint32) >> 16).astype(np.uint16).reshape(shape)
+    return spec, tensors
+
+
+def qwen_twin(Q, S, Wt, tag, W, H, G, hd, ff, V, P, B, steps, prompts, prefill_iters, max_ctx):
+    """The Qwen decoder (GQA, dense SwiGLU) with 4 layers at the given sizes through the same bench shapes."""
+    qs = S.ModelSpec(f"qwen-like-{tag}", 4, W, H, G, hd, ff, V, False, True, False, 1e-6)
+    qe = Q.Engine(qs, max_ctx=max_ctx).init_synthetic(Wt.SynthParams(seed=0))
+    qb = qe.batch(B, max_ctx)
+    qb.prefill(0, prompts[0])
+    tq = []
+    for _ in range(prefill_iters):
+        qe.sync()
+        t0 = time.perf_counter()
+        qb.prefill(0, prompts[0])
+        qe.sync()
+        tq.append(time.perf_counter() - t0)
+    for s_ in range(1, B):
+        qb.prefill(s_, prompts[s_])
+    qb.decode(8, want_ids=False)
+    qe.sync()
+    t0 = time.perf_counter()
+    qb.decode(steps, want_ids=False)
+    qe.sync()
+    dq = time.perf_counter() - t0
+    kern = {}
+    for name, which in (("gate_up", 0), ("down", 1), ("qkv", 2), ("o", 3), ("attention", 5)):
+        us, by = qb.time_kernel(which, 20)
+        kern[name] = {"us": round(us, 2), "GBps": round(by / us / 1e3, 1)}
+    out = {"model": f"{qs.n_layers} layers, hidden {qs.hidden}, {qs.n_heads}/{qs.n_kv_heads} heads of {qs.head_dim}, ffn {qs.ffn}",
+           "decode_tok_s": round(B * steps / dq, 1), "ms_per_step": round(dq * 1e3 / steps, 4),
+           "prefill_tok_s": round(P / float(np.median(tq)), 1), "prefill_ms": round(float(np.median(tq)) * 1e3, 3),
+           "prefill_tflops": round(qs.prefill_flops(P) / float(np.median(tq)) / 1e12, 2), "decode_kernels_B%d" % B: kern}
+    qb.close()
+    qe.close()
+    return out
+
+
+def run_nodutar(a):
+    """Prefill (one step of P tokens) and decode (B single-token entries a step at context ~P) of a Nodutar model,
+    per-stage hipEvent times at both shapes, and the Qwen decoder at equal sizes."""
+    import qwen_inference_engine_amd as Q
+    from qwen_inference_engine_amd import spec as S, weights as Wt
+    W, H, G, hd, rot, blk, RH, rd, rv, E, top, eff, V = NODUTAR_SIZES[a.nodutar]
+    P, B, steps = a.prompt, max(a.batch, 8), min(a.steps, 128)
+    max_ctx = P + steps + 80
+    spec, tensors = nodutar_model(S, a.nodutar)
+    out = {"metric": "nodutar_decode_tokens_per_sec", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16",
+           "data": "synthetic (random weights, random token ids)", "higher_is_better": True,
+           "config": {"model": spec.name, "sizes": dict(zip(("width", "heads", "kv_heads", "head_dim", "rot_dims", "block",
+                                                             "rec_heads", "rec_dim", "rec_vdim", "experts", "top", "expert_ff",
+                                                             "vocab"), NODUTAR_SIZES[a.nodutar])),
+                      "layers": 4, "prompt": P, "decode_batch": B, "decode_steps": steps}}
+    eng = Q.Engine(spec, max_ctx=max_ctx).load_tensors(tensors)
+    del tensors
+    b = eng.batch(B, max_ctx, page_tokens=64)
+    rng = np.random.default_rng(1)
+    prompts = rng.integers(0, V, size=(B, P), dtype=np.int32)
+    ts = []
+    for it in range(1 + a.prefill_iters):
+        t0 = time.perf_counter()
+        b.step([(0, prompts[0])], [P - 1], fetch=False)
+        ts.append(time.perf_counter() - t0)
+        if it < a.prefill_iters:
+            b.release(0)
+    t_pf = float(np.median(ts[1:]))
+    stages = {"prefill": {}, "decode": {}}
+    n_in = H * hd + 2 * G * hd + RH * (2 * rd + rv)
+
+    def stage_times(tag, rows, ctx):
+        st = stages[tag]
+        st["block_attention_us"] = round(b.time_stage(1, 0, 10), 2)
+        st["causal_attention_us"] = round(b.time_stage(1, 1, 10), 2)
+        st["mixer_products_us"] = round(b.time_stage(2, 0, 10), 2)
+        st["routed_ff_us"] = round(b.time_stage(3, 0, 10), 2)
+        st["recurrence_us"] = round(b.time_stage(4, 0, 10), 2)
+        # keys a query sees: its block so far / everything so far (prefill: on average half of that)
+        kb = min(ctx, blk) / 2.0 if tag == "prefill" else (ctx % blk) + 1
+        kc = ctx / (2.0 if tag == "prefill" else 1.0)
+        st["block_attention_tflops"] = round(4.0 * rows * H * kb * hd / st["block_attention_us"] / 1e6, 2)
+        st["causal_attention_tflops"] = round(4.0 * rows * H * kc * hd / st["causal_attention_us"] / 1e6, 2)
+        st["mixer_products_tflops"] = round(2.0 * rows * W * (n_in + H * hd + RH * rv) / st["mixer_products_us"] / 1e6, 2)
+        st["routed_ff_tflops"] = round(2.0 * rows * top * 3 * W * eff / st["routed_ff_us"] / 1e6, 2)
+        st["recurrence_gflops_fp32"] = round(4.0 * rows * RH * rd * rv / st["recurrence_us"] / 1e3, 1)
+        if tag == "decode":
+            st["causal_attention_GBps"] = round(rows * ctx * 2 * G * hd * 2 / st["causal_attention_us"] / 1e3, 1)
+            st["recurrence_state_GBps"] = round(rows * RH * rd * rv * 4 * 2 / st["recurrence_us"] / 1e3, 1)
+            st["mixer_products_GBps"] = round(W * (n_in + H * hd + RH * rv) * 2 / st["mixer_products_us"] / 1e3, 1)
+        st["layer_stack_us"] = round(b.time_stage(0, 0, 5), 2)
+    stage_times("prefill", P, P)
+    b.release(0)
+    for s_ in range(B):
+        for c0 in range(0, P, 512):
+            b.step([(s_, prompts[s_][c0:c0 + 512])], [], fetch=False)
+    toks = rng.integers(0, V, size=(steps + 8, B), dtype=np.int32)
+    for i in range(8):
+        b.step([(s_, [toks[i][s_]]) for s_ in range(B)], range(B), fetch=False)
+    t0 = time.perf_counter()
+    for i in range(8, 8 + steps):
+        b.step([(s_, [toks[i][s_]]) for s_ in range(B)], range(B), fetch=False)
+        b.step_sample()
+    dt = time.perf_counter() - t0
+    stage_times("decode", B, P)
+    out.update(value=round(B * steps / dt, 1), steps=steps, warmup=8, ms_per_step=round(dt * 1e3 / steps, 4),
+               prefill_tok_s=round(P / t_pf, 1), prefill_ms=round(t_pf * 1e3, 3),
+               prefill_tflops=round(spec.step_flops(P, P // 2) / t_pf / 1e12, 2), stages=stages, vs_baseline=None)
+    b.close()
+    eng.close()
+    out["qwen_equal_size"] = qwen_twin(Q, S, Wt, a.nodutar, W, H, G, hd, 2 * top * eff, V, P, B, steps, prompts, a.prefill_iters,
+                                       max_ctx)
+    print(json.dumps(out), flush=True)
+    return 0
 
 
 def run_layered(a):
