@@ -106,6 +106,9 @@ struct LayeredBatch {
     int64_t qgroups_cap = 0;
     int n_qgroups = 0;
     std::vector<int4> h_qgroups;
+    bool v_transposed = false;        // bf16 K / V caches on the matrix-core attention: V rows stored [kv_heads][vdim][page_tokens]
+    float *gpart_o = nullptr, *gpart_ml = nullptr;   // its key-split partials
+    int64_t gpart_cap = 0;            // (group, tile, split) units they hold
     int64_t cap = 0, want_cap = 0;
     float *stack = nullptr, *x = nullptr, *proj = nullptr, *qabs = nullptr, *olat = nullptr, *ov = nullptr, *mix = nullptr,
           *y = nullptr, *gu = nullptr, *act = nullptr, *ffo = nullptr, *xg = nullptr, *yd = nullptr, *score = nullptr,
@@ -143,7 +146,7 @@ struct LayeredBatch {
     int64_t steps = 0;
     bool keep_on = false;
     // per-row maxima over the layers (scratch sizing)
-    int64_t m_in = 0, m_hr = 0, m_hv = 0, m_gu = 0, m_act = 0, m_top = 0, m_e = 0, m_r = 0;
+    int64_t m_in = 0, m_hr = 0, m_hv = 0, m_gu = 0, m_act = 0, m_top = 0, m_e = 0, m_r = 0, m_vd = 0;
 };
 
 static inline float bf16_to_float(uint16_t h) {
@@ -732,6 +735,7 @@ static lay::GqaAttnP gqa_attn_params(qie_batch* b, int r) {
     p.cache = cache_of(b);
     p.k_off = s->layer_off[r];
     p.v_off = s->v_off[r];
+    p.v_transposed = s->v_transposed;
     p.out_scale = L.d.mixer == QIE_MIXER_GQA_RECURRENT ? L.d.gqa_scale : 1.0f;
     p.out = s->ov; p.out_bf = s->ov_bf; p.ld_out = L.n_cat; p.out_col = 0;
     return p;
@@ -768,6 +772,7 @@ static int enq_gqa_post(qie_batch* b, int r, int T) {
     p.cache = cache_of(b);
     p.k_off = s->layer_off[r];
     p.v_off = s->v_off[r];
+    p.v_transposed = s->v_transposed;
     return lay::gqa_post(p, m->f32, T, e->stream);
 }
 
@@ -775,8 +780,29 @@ static int enq_gqa_attention(qie_batch* b, int r, int T) {
     const qie_engine* e = b->e;
     LayeredBatch* s = b->lb;
     const lay::GqaAttnP p = gqa_attn_params(b, r);
-    if (!e->lm->f32 && s->n_qgroups > 0 && lay::gqa_attention_mfma_fits(p.dim, p.vdim)) {
-        lay::GqaAttnMfmaP q{p, s->d_qgroups, s->n_qgroups};
+    if (s->v_transposed && s->n_qgroups > 0) {
+        // enough key splits to fill the chip when the step has few rows (decoding)
+        const int tiles = (p.heads + 3) / 4 * 4;
+        const int64_t waves = (int64_t)s->n_qgroups * p.heads;
+        const int max_blocks = (p.mask == QIE_MASK_CAUSAL ? b->max_ctx : std::min(b->max_ctx, p.mask_size)) / 32 + 2;
+        const int S = (int)std::max<int64_t>(1, std::min<int64_t>({2048 / waves, max_blocks / 2, 32}));
+        const int64_t units = (int64_t)s->n_qgroups * tiles * S;
+        if (S > 1 && units > s->gpart_cap) {
+            hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+            QIE_REQUIRE(hipStreamIsCapturing(e->stream, &cs) == hipSuccess && cs == hipStreamCaptureStatusNone,
+                        "gqa attention: scratch growth inside a capture");
+            QIE_HIP(hipStreamSynchronize(e->stream));
+            drop_graphs(s);
+            if (s->gpart_o) hipFree(s->gpart_o);
+            if (s->gpart_ml) hipFree(s->gpart_ml);
+            s->gpart_o = s->gpart_ml = nullptr;
+            s->gpart_cap = 0;
+            const int64_t cap = (units + 255) / 256 * 256;
+            QIE_TRY(dmalloc((void**)&s->gpart_o, (size_t)cap * 16 * s->m_vd * 4));
+            QIE_TRY(dmalloc((void**)&s->gpart_ml, (size_t)cap * 16 * 2 * 4));
+            s->gpart_cap = cap;
+        }
+        lay::GqaAttnMfmaP q{p, s->d_qgroups, s->n_qgroups, S, s->gpart_o, s->gpart_ml};
         return lay::gqa_attention_mfma(q, e->stream);
     }
     return lay::gqa_attention(p, e->lm->f32, T, e->stream);
@@ -1088,6 +1114,14 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
         if (m->L[i].d.mixer != QIE_MIXER_LATENT_ATTENTION ||
             !lay::latent_attention_mfma_fits(m->L[i].d.kv_rank, m->L[i].d.rot_dim))
             s->interleaved = false;
+    // bf16 grouped-query caches whose every layer fits the matrix-core attention store V transposed
+    s->v_transposed = !m->f32;
+    for (int i = 0; i < m->a.n_layers; i++) {
+        const qie_layer_desc& d = m->L[i].d;
+        if (d.mixer == QIE_MIXER_LATENT_ATTENTION || !lay::gqa_attention_mfma_fits(d.gqa.dim, d.gqa.vdim, page_tokens))
+            s->v_transposed = false;
+        if (d.mixer != QIE_MIXER_LATENT_ATTENTION) s->m_vd = std::max<int64_t>(s->m_vd, d.gqa.vdim);
+    }
     int64_t off = 0;
     for (int r = 0; r < n_runs; r++) {
         const int i = m->runs[r].layer;
@@ -1184,7 +1218,7 @@ void layered_batch_destroy(qie_batch* b) {
     if (!s) return;
     lb_free(s);
     void* ps[] = {s->want, s->xn, s->logits, s->logits_bf, s->d_ids, s->d_step, s->d_groups, s->part_o, s->part_ml, s->xn_bf,
-                  s->state, s->d_ent, s->d_qgroups};
+                  s->state, s->d_ent, s->d_qgroups, s->gpart_o, s->gpart_ml};
     for (void* p : ps)
         if (p) hipFree(p);
     if (s->h_stage) hipHostFree(s->h_stage);

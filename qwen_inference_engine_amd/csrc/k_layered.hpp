@@ -125,6 +125,7 @@ struct GqaPostP {
     const float* vrope_sin;
     LatentCache cache;
     int64_t k_off, v_off;
+    int v_transposed;         // V rows of a page stored [kv_heads][vdim][page_tokens]
 };
 int gqa_post(const GqaPostP& p, bool cache_f32, int T, hipStream_t st);
 
@@ -149,6 +150,7 @@ struct GqaAttnP {
     const float* vrope_sin;
     LatentCache cache;
     int64_t k_off, v_off;
+    int v_transposed;
     float out_scale;
     float* out;
     uint16_t* out_bf;
@@ -156,14 +158,22 @@ struct GqaAttnP {
     int out_col;
 };
 int gqa_attention(const GqaAttnP& p, bool cache_f32, int T, hipStream_t st);
-// The matrix-core form for bf16 caches (dim and vdim multiples of 32 up to 256): one wave per 16
-// consecutive rows of one entry and head.  groups: {first packed row, rows, slot, first position}.
+// The matrix-core form for bf16 caches whose V rows are stored transposed (v_transposed: inside a
+// page [kv_heads][vdim][page_tokens], so that 4 keys of one value coordinate are one 8-byte load;
+// page_tokens a multiple of 32), dim a multiple of 32 and vdim of 16, both up to 256.  A wave takes
+// up to 16 (token, head) columns of one slot that share a key head: 16 consecutive tokens of one
+// head, or - for groups of few tokens - the heads of one key head per token.  groups: {first
+// packed row, tokens (<= 16), slot, first position}.  S > 1 splits every wave's keys S ways
+// (decoding: few columns, many keys); the partial sums meet in a second pass.  part_o
+// [groups * tiles * S][16][vdim], part_ml [...][16][2] floats of scratch (tiles = 4 * ceil(heads / 4)).
 struct GqaAttnMfmaP {
     GqaAttnP a;
     const int4* groups;
-    int n_groups;
+    int n_groups, S;
+    float* part_o;
+    float* part_ml;
 };
-bool gqa_attention_mfma_fits(int dim, int vdim);
+bool gqa_attention_mfma_fits(int dim, int vdim, int page_tokens);
 int gqa_attention_mfma(const GqaAttnMfmaP& p, hipStream_t st);
 
 // ------------------------------------------------------------------ gated linear recurrence

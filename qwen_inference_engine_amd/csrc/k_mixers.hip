@@ -92,7 +92,12 @@ __global__ __launch_bounds__(256) void gqa_post_kernel(GqaPostP p) {
     const int pt = pos % p.cache.page_tokens;
     const int H = p.heads, G = p.kv_heads, dim = p.dim, vdim = p.vdim;
     TC* krow = (TC*)p.cache.pool + pb + p.k_off + (int64_t)pt * G * dim;
-    TC* vrow = (TC*)p.cache.pool + pb + p.v_off + (int64_t)pt * G * vdim;
+    // value coordinate i of key head g: row-major rows, or one column of the page's transposed block
+    TC* vbase = (TC*)p.cache.pool + pb + p.v_off;
+    const int PT = p.cache.page_tokens;
+    auto vidx = [&](int g, int i) -> int64_t {
+        return p.v_transposed ? ((int64_t)g * vdim + i) * PT + pt : ((int64_t)pt * G + g) * vdim + i;
+    };
     const float* cs = p.rope_cos + (int64_t)pos * (p.rot_dims / 2);
     const float* sn = p.rope_sin + (int64_t)pos * (p.rot_dims / 2);
     for (int h0 = 0; h0 < H + G; h0 += 4) {
@@ -108,7 +113,7 @@ __global__ __launch_bounds__(256) void gqa_post_kernel(GqaPostP p) {
             }
             ss = wsum(ss);
             if (!is_q && p.v_col < 0)   // the value is the key as projected
-                for (int i = lane; i < dim; i += 64) stc<TC>(vrow, (int64_t)(hh - H) * dim + i, buf[i]);
+                for (int i = lane; i < dim; i += 64) stc<TC>(vbase, vidx(hh - H, i), buf[i]);
             if (p.qk_norm) {
                 const float inv = 1.0f / sqrtf(ss / (float)dim + p.eps);
                 const float* w = p.qk_norm == 1 ? (is_q ? p.qn_w : p.kn_w) : nullptr;
@@ -137,7 +142,7 @@ __global__ __launch_bounds__(256) void gqa_post_kernel(GqaPostP p) {
         __syncthreads();
         if (on)
             for (int i = lane; i < vdim; i += 64)
-                stc<TC>(vrow, (int64_t)g * vdim + i, p.rot_values ? turned(buf, i, vdim, p.rot_layout, vcs, vsn, 1.f) : buf[i]);
+                stc<TC>(vbase, vidx(g, i), p.rot_values ? turned(buf, i, vdim, p.rot_layout, vcs, vsn, 1.f) : buf[i]);
         __syncthreads();
     }
 }
@@ -225,13 +230,15 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(GqaAttnP p) {
         for (int i = 0; i < GA_MAXV; i++) acc[i] *= alpha;
         for (int jj = 0; jj < nk; jj++) {
             const int j = j0 + jj;
-            const TC* v = (const TC*)p.cache.pool + page_base(p.cache, slot, j) + p.v_off +
-                          ((int64_t)(j % p.cache.page_tokens) * G + g) * vdim;
+            const int pt = j % p.cache.page_tokens;
+            const TC* v = (const TC*)p.cache.pool + page_base(p.cache, slot, j) + p.v_off;
             const float w = sc[jj];
 #pragma unroll
             for (int i = 0; i < GA_MAXV; i++) {
                 const int r = tid + i * 256;
-                if (r < vdim) acc[i] = fmaf(w, ldc<TC>(v, r), acc[i]);
+                if (r < vdim)
+                    acc[i] = fmaf(w, ldc<TC>(v, p.v_transposed ? ((int64_t)g * vdim + r) * p.cache.page_tokens + pt
+                                                                 : ((int64_t)pt * G + g) * vdim + r), acc[i]);
             }
         }
         __syncthreads();
@@ -267,8 +274,263 @@ int gqa_attention(const GqaAttnP& p, bool cache_f32, int T, hipStream_t st) {
     return 0;
 }
 
-bool gqa_attention_mfma_fits(int dim, int vdim) { return false; }
-int gqa_attention_mfma(const GqaAttnMfmaP& p, hipStream_t st) { return fail(-22, "gqa attention: no matrix-core form for these sizes"); }
+// ------------------------------------------------------------------ attention on the matrix cores
+// S^T = K Q^T per 32 keys (two 16 x 16 tiles, K rows as A fragments straight from the cache, the
+// queries as bf16 B fragments in registers), masks, bias and the running maximum / sum per
+// column in fp32 (a column's 32 scores live in 4 lanes), then O^T += V^T P^T with the softmax
+// weights as the B fragment in the order the score tiles left them: k-slot e of lane group g is
+// key 4g + e (e < 4) or 16 + 4g + e - 4, which the transposed V rows serve with two 8-byte loads.
+// No LDS, no barrier: waves of a workgroup are independent (they share key heads through the L1).
+typedef __bf16 gbf16x8_t __attribute__((ext_vector_type(8)));
+typedef float gf32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float xg_max(float v) {   // over the 4 lanes n, n + 16, n + 32, n + 48
+    v = fmaxf(v, __shfl_xor(v, 16, 64));
+    return fmaxf(v, __shfl_xor(v, 32, 64));
+}
+__device__ __forceinline__ float xg_sum(float v) {
+    v += __shfl_xor(v, 16, 64);
+    return v + __shfl_xor(v, 32, 64);
+}
+
+// heads of one key head that a group of n_tok tokens packs into its 16 columns
+__host__ __device__ __forceinline__ int heads_per_token(int n_tok, int H, int G) {
+    const int hpk = H / G;
+    return (hpk <= 16 && n_tok * hpk <= 16) ? hpk : 1;
+}
+
+// One column's finished value sums o[v] (v = v0 .. v0 + 3 of every 16-tile) -> out: turned back by
+// the column's position when asked, scaled, stored with the bf16 image.
+template <int DV>
+__device__ __forceinline__ void gqa_store(const GqaAttnP& a, const gf32x4_t* acc, float inv, int row, int hh, int qpos, int g) {
+    const int vdim = 16 * DV;
+    const int64_t o0 = (int64_t)row * a.ld_out + a.out_col + (int64_t)hh * vdim;
+    const float* cs = a.rot_values ? a.vrope_cos + (int64_t)qpos * (vdim / 2) : nullptr;
+    const float* sn = a.rot_values ? a.vrope_sin + (int64_t)qpos * (vdim / 2) : nullptr;
+#pragma unroll
+    for (int dv = 0; dv < DV; dv++) {
+        float o[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) o[j] = acc[dv][j] * inv;
+        const int v0 = 16 * dv + 4 * g;
+        if (a.rot_values) {
+            if (a.rot_layout == 1) {   // (v0, v0 + 1), (v0 + 2, v0 + 3): turned back = the angle negated
+#pragma unroll
+                for (int j = 0; j < 4; j += 2) {
+                    const float c = cs[(v0 + j) >> 1], s = sn[(v0 + j) >> 1];
+                    const float u = o[j], w = o[j + 1];
+                    o[j] = u * c + w * s;
+                    o[j + 1] = w * c - u * s;
+                }
+            } else {                   // v with v + vdim / 2: the partner sits DV / 2 tiles away in this lane
+                const bool low = dv < DV / 2;
+                const int dp = low ? dv + DV / 2 : dv - DV / 2;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const int pi = (low ? v0 : v0 - vdim / 2) + j;
+                    const float c = cs[pi], s = sn[pi];
+                    const float mine = acc[dv][j] * inv, other = acc[dp][j] * inv;
+                    o[j] = low ? mine * c + other * s : mine * c - other * s;
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float y = o[j] * a.out_scale;
+            a.out[o0 + v0 + j] = y;
+            if (a.out_bf) a.out_bf[o0 + v0 + j] = f2bf(y);
+        }
+    }
+}
+
+template <int DK, int DV>
+__global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(GqaAttnMfmaP P) {
+    const GqaAttnP& a = P.a;
+    constexpr int dim = 32 * DK, vdim = 16 * DV;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 4, n = lane & 15;
+    const int4 grp = P.groups[blockIdx.x];
+    const int n_tok = grp.y, slot = grp.z, pos0 = grp.w;
+    const int H = a.heads, G = a.kv_heads;
+    const int hpt = heads_per_token(n_tok, H, G);
+    const int tile = blockIdx.y * 4 + wave, h0 = tile * hpt;
+    if (h0 >= H) return;
+    const int tI = n / hpt, hh = h0 + n % hpt;
+    const bool valid = tI < n_tok;
+    const int tC = valid ? tI : n_tok - 1;
+    const int qpos = pos0 + tC, row = grp.x + tC;
+    const int kvh = h0 / (H / G);
+    // queries: B fragments (column n, k-slots 8g .. 8g + 7 of every 32 coordinates)
+    gbf16x8_t qf[DK];
+    {
+        const float* qr = a.proj + (int64_t)row * a.ld + a.q_col + hh * dim + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < DK; ks++) {
+            float x[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) x[i] = qr[32 * ks + i];
+            const uint4 u = make_uint4(pack2(x[0], x[1]), pack2(x[2], x[3]), pack2(x[4], x[5]), pack2(x[6], x[7]));
+            qf[ks] = __builtin_bit_cast(gbf16x8_t, u);
+        }
+    }
+    const int lo_q = first_visible(a.mask, a.mask_size, qpos);
+    const int kmin = first_visible(a.mask, a.mask_size, pos0), kmax = pos0 + n_tok - 1;
+    const int b0 = kmin >> 5, nb = (kmax >> 5) - b0 + 1;
+    const int S = P.S, z = blockIdx.z;
+    const int bs = b0 + (int)((int64_t)nb * z / S), be = b0 + (int)((int64_t)nb * (z + 1) / S);
+    const float b1 = a.r1 ? a.r1[hh] : 0.f, b2 = a.r1 ? a.r2[hh] : 0.f;
+    const int PT = a.cache.page_tokens;
+    const uint16_t* pool = (const uint16_t*)a.cache.pool;
+    const int32_t* tab = a.cache.table + (int64_t)slot * a.cache.max_pages;
+    float m_run = -1e30f, l_run = 0.f;
+    gf32x4_t acc[DV];
+#pragma unroll
+    for (int dv = 0; dv < DV; dv++) acc[dv] = gf32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int kb = bs; kb < be; kb++) {
+        const int key0 = kb << 5;
+        const int64_t pb = (int64_t)tab[key0 / PT] * a.cache.page_stride;
+        const int tok0 = key0 % PT;
+        gf32x4_t sacc[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+            sacc[tt] = gf32x4_t{0.f, 0.f, 0.f, 0.f};
+            const uint16_t* kr = pool + pb + a.k_off + ((int64_t)(tok0 + 16 * tt + n) * G + kvh) * dim + 8 * g;
+#pragma unroll
+            for (int ks = 0; ks < DK; ks++) {
+                const uint4 kf = *reinterpret_cast<const uint4*>(kr + 32 * ks);
+                sacc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(gbf16x8_t, kf), qf[ks], sacc[tt], 0, 0, 0);
+            }
+        }
+        float s[8];
+        bool vis[8];
+        float bm = -1e30f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int kj = key0 + 16 * (e >> 2) + 4 * g + (e & 3);
+            vis[e] = valid && kj >= lo_q && kj <= qpos;
+            float x = sacc[e >> 2][e & 3] * a.scale;
+            if (a.r1) x -= b1 * log1pf(b2 * (float)max(qpos - kj, 0));
+            s[e] = vis[e] ? x : -1e30f;
+            bm = fmaxf(bm, s[e]);
+        }
+        bm = xg_max(bm);
+        const float m_new = fmaxf(m_run, bm);
+        const float alpha = expf(m_run - m_new);
+        float ls = 0.f, pv[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            pv[e] = vis[e] ? expf(s[e] - m_new) : 0.f;
+            ls += pv[e];
+        }
+        ls = xg_sum(ls);
+        l_run = l_run * alpha + ls;
+        m_run = m_new;
+        const uint4 pu = make_uint4(pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]), pack2(pv[6], pv[7]));
+        const gbf16x8_t pf = __builtin_bit_cast(gbf16x8_t, pu);
+        const uint16_t* vr = pool + pb + a.v_off + ((int64_t)kvh * vdim + n) * PT + tok0 + 4 * g;
+#pragma unroll
+        for (int dv = 0; dv < DV; dv++) {
+            const uint2 v0 = *reinterpret_cast<const uint2*>(vr + (int64_t)16 * dv * PT);
+            const uint2 v1 = *reinterpret_cast<const uint2*>(vr + (int64_t)16 * dv * PT + 16);
+            const uint4 vu = make_uint4(v0.x, v0.y, v1.x, v1.y);
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[dv][j] *= alpha;
+            acc[dv] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(gbf16x8_t, vu), pf, acc[dv], 0, 0, 0);
+        }
+    }
+    if (S == 1) {
+        if (valid) gqa_store<DV>(a, acc, 1.0f / l_run, row, hh, qpos, g);
+        return;
+    }
+    const int64_t unit = ((int64_t)blockIdx.x * (gridDim.y * 4) + tile) * S + z;
+    float* po = P.part_o + (unit * 16 + n) * vdim + 4 * g;
+#pragma unroll
+    for (int dv = 0; dv < DV; dv++) *reinterpret_cast<float4*>(po + 16 * dv) = make_float4(acc[dv][0], acc[dv][1], acc[dv][2], acc[dv][3]);
+    if (g == 0) {
+        P.part_ml[(unit * 16 + n) * 2] = m_run;
+        P.part_ml[(unit * 16 + n) * 2 + 1] = l_run;
+    }
+}
+
+// Second pass of a split launch: one wave per (group, tile), the same lane layout as the first.
+template <int DV>
+__global__ __launch_bounds__(256) void gqa_attn_combine_kernel(GqaAttnMfmaP P, int tiles) {
+    const GqaAttnP& a = P.a;
+    constexpr int vdim = 16 * DV;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 4, n = lane & 15;
+    const int4 grp = P.groups[blockIdx.x];
+    const int n_tok = grp.y, pos0 = grp.w;
+    const int hpt = heads_per_token(n_tok, a.heads, a.kv_heads);
+    const int tile = blockIdx.y * 4 + wave, h0 = tile * hpt;
+    if (h0 >= a.heads) return;
+    const int tI = n / hpt, hh = h0 + n % hpt;
+    if (tI >= n_tok) return;
+    const int64_t u0 = ((int64_t)blockIdx.x * tiles + tile) * P.S;
+    float M = -1e30f;
+    for (int z = 0; z < P.S; z++) M = fmaxf(M, P.part_ml[((u0 + z) * 16 + n) * 2]);
+    float L = 0.f;
+    gf32x4_t acc[DV];
+#pragma unroll
+    for (int dv = 0; dv < DV; dv++) acc[dv] = gf32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int z = 0; z < P.S; z++) {
+        const float l = P.part_ml[((u0 + z) * 16 + n) * 2 + 1];
+        if (l == 0.f) continue;   // this part saw no key of the column
+        const float w = expf(P.part_ml[((u0 + z) * 16 + n) * 2] - M);
+        L += l * w;
+        const float* po = P.part_o + ((u0 + z) * 16 + n) * vdim + 4 * g;
+#pragma unroll
+        for (int dv = 0; dv < DV; dv++) {
+            const float4 o = *reinterpret_cast<const float4*>(po + 16 * dv);
+            acc[dv][0] += o.x * w; acc[dv][1] += o.y * w; acc[dv][2] += o.z * w; acc[dv][3] += o.w * w;
+        }
+    }
+    gqa_store<DV>(a, acc, 1.0f / L, grp.x + tI, hh, pos0 + tI, g);
+}
+
+bool gqa_attention_mfma_fits(int dim, int vdim, int page_tokens) {
+    auto one_of = [](int x, int unit) { return x == unit || x == 2 * unit || x == 4 * unit || x == 8 * unit; };
+    return one_of(dim, 32) && one_of(vdim, 32) && page_tokens % 32 == 0;
+}
+
+template <int DK>
+static int gqa_mfma_launch(const GqaAttnMfmaP& p, dim3 grid, hipStream_t st) {
+    const int tiles = (int)grid.y * 4;
+    dim3 cg(grid.x, grid.y, 1);
+    switch (p.a.vdim / 32) {
+        case 1:
+            hipLaunchKernelGGL((gqa_attn_mfma_kernel<DK, 2>), grid, dim3(256), 0, st, p);
+            if (p.S > 1) hipLaunchKernelGGL(gqa_attn_combine_kernel<2>, cg, dim3(256), 0, st, p, tiles);
+            break;
+        case 2:
+            hipLaunchKernelGGL((gqa_attn_mfma_kernel<DK, 4>), grid, dim3(256), 0, st, p);
+            if (p.S > 1) hipLaunchKernelGGL(gqa_attn_combine_kernel<4>, cg, dim3(256), 0, st, p, tiles);
+            break;
+        case 4:
+            hipLaunchKernelGGL((gqa_attn_mfma_kernel<DK, 8>), grid, dim3(256), 0, st, p);
+            if (p.S > 1) hipLaunchKernelGGL(gqa_attn_combine_kernel<8>, cg, dim3(256), 0, st, p, tiles);
+            break;
+        default:
+            hipLaunchKernelGGL((gqa_attn_mfma_kernel<DK, 16>), grid, dim3(256), 0, st, p);
+            if (p.S > 1) hipLaunchKernelGGL(gqa_attn_combine_kernel<16>, cg, dim3(256), 0, st, p, tiles);
+            break;
+    }
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+int gqa_attention_mfma(const GqaAttnMfmaP& p, hipStream_t st) {
+    const GqaAttnP& a = p.a;
+    QIE_REQUIRE(gqa_attention_mfma_fits(a.dim, a.vdim, a.cache.page_tokens) && a.v_transposed,
+                "gqa attention: sizes %d / %d, pages of %d tokens do not fit the matrix-core form", a.dim, a.vdim, a.cache.page_tokens);
+    QIE_REQUIRE(p.n_groups > 0 && p.S >= 1 && (p.S == 1 || (p.part_o && p.part_ml)), "gqa attention: bad launch");
+    QIE_REQUIRE(a.heads % a.kv_heads == 0, "gqa attention: %d query heads over %d key heads", a.heads, a.kv_heads);
+    dim3 grid((unsigned)p.n_groups, (unsigned)((a.heads + 3) / 4), (unsigned)p.S);
+    switch (a.dim / 32) {
+        case 1: return gqa_mfma_launch<1>(p, grid, st);
+        case 2: return gqa_mfma_launch<2>(p, grid, st);
+        case 4: return gqa_mfma_launch<4>(p, grid, st);
+        default: return gqa_mfma_launch<8>(p, grid, st);
+    }
+}
 
 // ------------------------------------------------------------------ gated linear recurrence
 // One block per (head, entry, 64 value columns).  A thread owns one column of SR state rows in

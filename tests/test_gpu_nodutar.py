@@ -280,14 +280,16 @@ def test_other_sizes(model):
     assert rel(feed(m, 0, toks, [33, 2, 20]), m.ref(toks)) < REL32
 
 
-@pytest.mark.parametrize("hd,size", [(32, 21), (64, 40), (128, 70)], ids=["hd32", "hd64", "hd128"])
-def test_bf16_matrix_shapes(model, hd, size):
-    """Sizes that take the bf16 matrix kernels: whole prompts, portions and single tokens against the oracle,
-    beside another request, with more than 256 routed rows in one step."""
+@pytest.mark.parametrize("hd,size,page", [(32, 21, 32), (64, 40, 64), (128, 70, 32), (64, 33, 16)],
+                         ids=["hd32", "hd64", "hd128", "hd64-page16"])
+def test_bf16_matrix_shapes(model, hd, size, page):
+    """Sizes that take the bf16 matrix kernels (pages of 32 or more tokens: attention on the matrix cores over
+    transposed value rows, key splits while decoding; pages of 16: the plain attention): whole prompts, portions
+    and single tokens against the oracle, beside another request, with more than 256 routed rows in one step."""
     layers = [par(heads=4, kv_heads=2, dim=hd, vdim=hd, rot_dims=hd // 2, size=size, scale=0.5, rheads=2, rdim=32, rvdim=64,
                   mlp=("moe", 32, 4, 2)),
               dist(heads=4, kv_heads=1, dim=hd, scale=1.0, mlp=("moe", 96, 4, 2))]
-    m = model(layers, seed=hd, vocab=160, width=64, dtype="bfloat16", page_tokens=16, max_ctx=512, loop=(0, 1, 2))
+    m = model(layers, seed=hd, vocab=160, width=64, dtype="bfloat16", page_tokens=page, max_ctx=512, loop=(0, 1, 2))
     toks = m.tokens(150)
     want = m.ref(toks)
     assert rel_most(O.forward(with_mask(m.cfg, 1), m.T, toks), want, 0.97) > 2 * REL16
