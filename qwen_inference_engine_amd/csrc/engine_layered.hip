@@ -106,6 +106,14 @@ struct LayeredBatch {
     int64_t qgroups_cap = 0;
     int n_qgroups = 0;
     std::vector<int4> h_qgroups;
+    // recurrent mixers, long entries: pieces of kScanPiece rows scanned side by side (lay::gated_carry)
+    int4 *d_chunks = nullptr, *d_spans = nullptr;
+    int64_t chunks_cap = 0;
+    int n_chunks = 0, max_count = 0;
+    std::vector<int4> h_chunks, h_spans;
+    float *s_loc = nullptr, *s_in = nullptr, *s_decay = nullptr;
+    int64_t scan_cap = 0;             // pieces the three buffers hold
+    int64_t m_state = 0, m_hd = 0;    // largest state / gate row count of a layer run
     bool v_transposed = false;        // bf16 K / V caches on the matrix-core attention: V rows stored [kv_heads][vdim][page_tokens]
     float *gpart_o = nullptr, *gpart_ml = nullptr;   // its key-split partials
     int64_t gpart_cap = 0;            // (group, tile, split) units they hold
@@ -808,6 +816,9 @@ static int enq_gqa_attention(qie_batch* b, int r, int T) {
     return lay::gqa_attention(p, e->lm->f32, T, e->stream);
 }
 
+// Rows of an entry above which the recurrence runs in pieces; rows per piece.
+constexpr int kScanLong = 128, kScanPiece = 64;
+
 static int enq_recurrence(qie_batch* b, int r, int T) {
     const qie_engine* e = b->e;
     const LayeredModel* m = e->lm;
@@ -821,8 +832,26 @@ static int enq_recurrence(qie_batch* b, int r, int T) {
     p.f_bias = L.rec_fb; p.lower = L.rec_lower;
     p.state = s->state; p.slot_stride = s->slot_state; p.state_off = s->state_off[r];
     p.out = s->olat;
+    if (s->max_count > kScanLong && s->s_loc) {
+        const int64_t n = (int64_t)c.heads * c.dim * c.vdim;
+        lay::GatedScanP a = p;       // pieces from zero states: local outputs, end states, gate products
+        a.entries = s->d_chunks; a.n_entries = s->n_chunks;
+        a.state = s->s_loc; a.slot_stride = n; a.state_off = 0;
+        a.decay = s->s_decay;
+        QIE_TRY(lay::gated_scan(a, e->stream));
+        lay::GatedCarryP k{s->d_spans, s->n_ent, c.heads, c.dim, c.vdim, s->s_loc, s->s_decay, s->s_in, s->state, s->slot_state,
+                           s->state_off[r]};
+        QIE_TRY(lay::gated_carry(k, e->stream));
+        a.state = s->s_in;           // the incoming states' share of every row, summed in the head norm
+        a.mode = 1;
+        a.decay = nullptr;
+        a.out = s->qabs;
+        QIE_TRY(lay::gated_scan(a, e->stream));
+        return lay::head_norm_rows(s->olat, s->qabs, L.rec_norm, m->a.norm_eps, L.d.rec_scale, c.heads, c.vdim, T, s->ov, s->ov_bf,
+                                   L.n_cat, L.cat_rec, e->stream);
+    }
     QIE_TRY(lay::gated_scan(p, e->stream));
-    return lay::head_norm_rows(s->olat, L.rec_norm, m->a.norm_eps, L.d.rec_scale, c.heads, c.vdim, T, s->ov, s->ov_bf, L.n_cat,
+    return lay::head_norm_rows(s->olat, nullptr, L.rec_norm, m->a.norm_eps, L.d.rec_scale, c.heads, c.vdim, T, s->ov, s->ov_bf, L.n_cat,
                                L.cat_rec, e->stream);
 }
 
@@ -1137,6 +1166,8 @@ int layered_batch_create(qie_engine* e, int32_t batch, int32_t max_ctx, int32_t 
             if (rv) {
                 s->state_off[r] = s->slot_state;
                 s->slot_state += (int64_t)d.rec.heads * d.rec.dim * d.rec.vdim;
+                s->m_state = std::max<int64_t>(s->m_state, (int64_t)d.rec.heads * d.rec.dim * d.rec.vdim);
+                s->m_hd = std::max<int64_t>(s->m_hd, (int64_t)d.rec.heads * d.rec.dim);
             }
             s->m_in = std::max<int64_t>(s->m_in, m->L[i].n_in);
             s->m_hr = std::max<int64_t>(s->m_hr, rv);
@@ -1218,7 +1249,7 @@ void layered_batch_destroy(qie_batch* b) {
     if (!s) return;
     lb_free(s);
     void* ps[] = {s->want, s->xn, s->logits, s->logits_bf, s->d_ids, s->d_step, s->d_groups, s->part_o, s->part_ml, s->xn_bf,
-                  s->state, s->d_ent, s->d_qgroups, s->gpart_o, s->gpart_ml};
+                  s->state, s->d_ent, s->d_qgroups, s->gpart_o, s->gpart_ml, s->d_chunks, s->d_spans, s->s_loc, s->s_in, s->s_decay};
     for (void* p : ps)
         if (p) hipFree(p);
     if (s->h_stage) hipHostFree(s->h_stage);
@@ -1455,6 +1486,38 @@ int qie_batch_step(qie_batch* b, int32_t n_entries, const int32_t* slots, const 
         QIE_HIP(hipMemcpyAsync(s->d_qgroups, s->h_qgroups.data(), s->h_qgroups.size() * sizeof(int4), hipMemcpyHostToDevice, st));
         s->n_ent = n_entries;
         s->n_qgroups = (int)s->h_qgroups.size();
+        s->max_count = 0;
+        for (int i = 0; i < n_entries; i++) s->max_count = std::max(s->max_count, (int)counts[i]);
+        if (s->slot_state > 0 && s->max_count > kScanLong) {
+            s->h_chunks.clear();
+            s->h_spans.clear();
+            for (const int4& en : s->h_ent) {
+                const int c0 = (int)s->h_chunks.size();
+                for (int k = 0; k < en.y; k += kScanPiece)
+                    s->h_chunks.push_back(int4{en.x + k, std::min(kScanPiece, en.y - k), (int)s->h_chunks.size(), 0});
+                s->h_spans.push_back(int4{c0, (int)s->h_chunks.size() - c0, en.z, en.w});
+            }
+            const int64_t nc = (int64_t)s->h_chunks.size();
+            if (nc > s->chunks_cap || nc > s->scan_cap) {
+                QIE_HIP(hipStreamSynchronize(st));
+                void* ps[] = {s->d_chunks, s->d_spans, s->s_loc, s->s_in, s->s_decay};
+                for (void* q : ps)
+                    if (q) hipFree(q);
+                s->d_chunks = s->d_spans = nullptr;
+                s->s_loc = s->s_in = s->s_decay = nullptr;
+                s->chunks_cap = s->scan_cap = 0;
+                const int64_t cap = (nc + 63) / 64 * 64;
+                QIE_TRY(dmalloc((void**)&s->d_chunks, (size_t)cap * sizeof(int4)));
+                QIE_TRY(dmalloc((void**)&s->d_spans, (size_t)std::max<int64_t>(b->B, n_entries) * sizeof(int4)));
+                QIE_TRY(dmalloc((void**)&s->s_loc, (size_t)cap * s->m_state * 4));
+                QIE_TRY(dmalloc((void**)&s->s_in, (size_t)cap * s->m_state * 4));
+                QIE_TRY(dmalloc((void**)&s->s_decay, (size_t)cap * s->m_hd * 4));
+                s->chunks_cap = s->scan_cap = cap;
+            }
+            QIE_HIP(hipMemcpyAsync(s->d_chunks, s->h_chunks.data(), s->h_chunks.size() * sizeof(int4), hipMemcpyHostToDevice, st));
+            QIE_HIP(hipMemcpyAsync(s->d_spans, s->h_spans.data(), s->h_spans.size() * sizeof(int4), hipMemcpyHostToDevice, st));
+            s->n_chunks = (int)nc;
+        }
     }
     QIE_HIP(hipMemcpyAsync(s->row_slot, hs, (size_t)T * 4, hipMemcpyHostToDevice, st));
     QIE_HIP(hipMemcpyAsync(s->row_pos, hs + R, (size_t)T * 4, hipMemcpyHostToDevice, st));

@@ -194,11 +194,36 @@ struct GatedScanP {
     float* state;
     int64_t slot_stride, state_off;
     float* out;
+    // mode 0: the recurrence itself (state read unless the entry starts at position 0, advanced,
+    // written back); decay (optional) receives the product of the entry's gates, [entries][heads][dim].
+    // mode 1: the state is only read, every row's q is scaled by the product of the gates from the
+    // entry's first row to this row, and out receives S^T q: the share of an incoming state in the
+    // outputs of rows that were scanned from a zero state (the caller adds the two).
+    int mode;
+    float* decay;
 };
 int gated_scan(const GatedScanP& p, hipStream_t st);
-// out[t, out_col + h * vdim + c] = scale * o[t, h, c] / sqrt(mean_c o^2 + eps) * w[c]
-int head_norm_rows(const float* o, const float* w, float eps, float scale, int heads, int vdim, int T, float* out, uint16_t* out_bf,
-                   int64_t ld_out, int out_col, hipStream_t st);
+// Long entries in pieces: `chunks` lists pieces {first packed row, rows, piece index, 0} in entry
+// order, `spans` one {first piece, pieces, slot, first position} per entry.  gated_scan (mode 0)
+// over the pieces from zero states gives piece-local outputs, end states s_loc [pieces][heads *
+// dim * vdim] and gate products; gated_carry walks an entry's pieces in order (s_in[c] = state
+// entering piece c, starting from the slot's state or zero; the slot's state = what leaves the
+// last piece); gated_scan (mode 1) over the pieces with s_in gives the incoming states' share.
+// Same sums as the row-by-row recurrence up to fp32 rounding.
+struct GatedCarryP {
+    const int4* spans;
+    int n_spans;
+    int heads, dim, vdim;
+    const float* s_loc;
+    const float* decay;
+    float* s_in;
+    float* state;
+    int64_t slot_stride, state_off;
+};
+int gated_carry(const GatedCarryP& p, hipStream_t st);
+// out[t, out_col + h * vdim + c] = scale * o[t, h, c] / sqrt(mean_c o^2 + eps) * w[c], o = o1 + o2 when o2
+int head_norm_rows(const float* o, const float* o2, const float* w, float eps, float scale, int heads, int vdim, int T, float* out,
+                   uint16_t* out_bf, int64_t ld_out, int out_col, hipStream_t st);
 // Rows of W: x = xin + rms(v) * (1 + wb) (when v) + add (when add); then (when wn)
 // h = rms(x) * (1 + wn) with its bf16 image.  xin may be x.
 int add_norm(float* x, const float* xin, const float* v, const float* wb, const float* add, const float* wn, float* h, uint16_t* h_bf,

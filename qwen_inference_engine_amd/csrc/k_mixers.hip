@@ -385,20 +385,42 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(GqaAttnMfmaP P) {
     gf32x4_t acc[DV];
 #pragma unroll
     for (int dv = 0; dv < DV; dv++) acc[dv] = gf32x4_t{0.f, 0.f, 0.f, 0.f};
+    // K fragments of a 32-key block: two 16-key tiles x DK steps of 32 coordinates; the next
+    // block's are loaded while this block is scored, the block's V fragments before its softmax
+    uint4 kf[2][DK], kn[2][DK];
+    auto load_k = [&](int kb, uint4 (&dst)[2][DK]) {
+        const int key0 = kb << 5;
+        const int64_t pb = (int64_t)tab[key0 / PT] * a.cache.page_stride;
+        const int tok0 = key0 % PT;
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+            const uint16_t* kr = pool + pb + a.k_off + ((int64_t)(tok0 + 16 * tt + n) * G + kvh) * dim + 8 * g;
+#pragma unroll
+            for (int ks = 0; ks < DK; ks++) dst[tt][ks] = *reinterpret_cast<const uint4*>(kr + 32 * ks);
+        }
+    };
+    if (bs < be) load_k(bs, kf);
     for (int kb = bs; kb < be; kb++) {
         const int key0 = kb << 5;
         const int64_t pb = (int64_t)tab[key0 / PT] * a.cache.page_stride;
         const int tok0 = key0 % PT;
+        uint2 vf[DV][2];
+        {
+            const uint16_t* vr = pool + pb + a.v_off + ((int64_t)kvh * vdim + n) * PT + tok0 + 4 * g;
+#pragma unroll
+            for (int dv = 0; dv < DV; dv++) {
+                vf[dv][0] = *reinterpret_cast<const uint2*>(vr + (int64_t)16 * dv * PT);
+                vf[dv][1] = *reinterpret_cast<const uint2*>(vr + (int64_t)16 * dv * PT + 16);
+            }
+        }
+        if (kb + 1 < be) load_k(kb + 1, kn);
         gf32x4_t sacc[2];
 #pragma unroll
         for (int tt = 0; tt < 2; tt++) {
             sacc[tt] = gf32x4_t{0.f, 0.f, 0.f, 0.f};
-            const uint16_t* kr = pool + pb + a.k_off + ((int64_t)(tok0 + 16 * tt + n) * G + kvh) * dim + 8 * g;
 #pragma unroll
-            for (int ks = 0; ks < DK; ks++) {
-                const uint4 kf = *reinterpret_cast<const uint4*>(kr + 32 * ks);
-                sacc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(gbf16x8_t, kf), qf[ks], sacc[tt], 0, 0, 0);
-            }
+            for (int ks = 0; ks < DK; ks++)
+                sacc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(gbf16x8_t, kf[tt][ks]), qf[ks], sacc[tt], 0, 0, 0);
         }
         float s[8];
         bool vis[8];
@@ -408,17 +430,17 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(GqaAttnMfmaP P) {
             const int kj = key0 + 16 * (e >> 2) + 4 * g + (e & 3);
             vis[e] = valid && kj >= lo_q && kj <= qpos;
             float x = sacc[e >> 2][e & 3] * a.scale;
-            if (a.r1) x -= b1 * log1pf(b2 * (float)max(qpos - kj, 0));
+            if (a.r1) x -= b1 * __logf(1.0f + b2 * (float)max(qpos - kj, 0));
             s[e] = vis[e] ? x : -1e30f;
             bm = fmaxf(bm, s[e]);
         }
         bm = xg_max(bm);
         const float m_new = fmaxf(m_run, bm);
-        const float alpha = expf(m_run - m_new);
+        const float alpha = __expf(m_run - m_new);
         float ls = 0.f, pv[8];
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            pv[e] = vis[e] ? expf(s[e] - m_new) : 0.f;
+            pv[e] = vis[e] ? __expf(s[e] - m_new) : 0.f;
             ls += pv[e];
         }
         ls = xg_sum(ls);
@@ -426,16 +448,17 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(GqaAttnMfmaP P) {
         m_run = m_new;
         const uint4 pu = make_uint4(pack2(pv[0], pv[1]), pack2(pv[2], pv[3]), pack2(pv[4], pv[5]), pack2(pv[6], pv[7]));
         const gbf16x8_t pf = __builtin_bit_cast(gbf16x8_t, pu);
-        const uint16_t* vr = pool + pb + a.v_off + ((int64_t)kvh * vdim + n) * PT + tok0 + 4 * g;
 #pragma unroll
         for (int dv = 0; dv < DV; dv++) {
-            const uint2 v0 = *reinterpret_cast<const uint2*>(vr + (int64_t)16 * dv * PT);
-            const uint2 v1 = *reinterpret_cast<const uint2*>(vr + (int64_t)16 * dv * PT + 16);
-            const uint4 vu = make_uint4(v0.x, v0.y, v1.x, v1.y);
+            const uint4 vu = make_uint4(vf[dv][0].x, vf[dv][0].y, vf[dv][1].x, vf[dv][1].y);
 #pragma unroll
             for (int j = 0; j < 4; j++) acc[dv][j] *= alpha;
             acc[dv] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(gbf16x8_t, vu), pf, acc[dv], 0, 0, 0);
         }
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+            for (int ks = 0; ks < DK; ks++) kf[tt][ks] = kn[tt][ks];
     }
     if (S == 1) {
         if (valid) gqa_store<DV>(a, acc, 1.0f / l_run, row, hh, qpos, g);
@@ -537,11 +560,16 @@ int gqa_attention_mfma(const GqaAttnMfmaP& p, hipStream_t st) {
 // registers; blockDim / 64 thread groups split the dim rows.  The entry's rows go through in
 // tiles: the tile's q, f (activations applied, fp32) and v are staged in LDS, every token then
 // costs SR multiply-adds per thread with no synchronisation; the groups' partial outputs meet in
-// LDS once a tile.  Rows beyond dim are padded with f = 1, q = 0 (their state stays 0).
+// LDS once a tile.  Rows beyond dim are padded with f = 1, q = 0 (their state stays 0).  mode 1
+// writes (not adds) its share to out: the caller passes a buffer of its own and sums later.
 constexpr int SR = 32;
 
-__global__ __launch_bounds__(1024) void gated_scan_kernel(GatedScanP p, int TT, int dimP) {
-    extern __shared__ float sm[];
+// TT rows per tile.  The next tile's projection values are loaded into registers while the
+// current tile is computed (a block is one to sixteen waves on a CU of its own: nothing else
+// would hide the loads), activated and stored to LDS once the tile is done.
+template <int TT, int MAXT>
+__global__ __launch_bounds__(MAXT) void gated_scan_kernel(GatedScanP p, int dimP) {
+    extern __shared__ __align__(16) float sm[];
     const int NG = blockDim.x >> 6;
     float* qs = sm;                       // [TT][dimP]
     float* fs = qs + TT * dimP;           // [TT][dimP]
@@ -556,43 +584,99 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(GatedScanP p, int TT, 
 #pragma unroll
     for (int r = 0; r < SR; r++) {
         const int d = d0 + r;
-        S[r] = (en.w > 0 && d < dim && cok) ? stp[(int64_t)d * vdim + c] : 0.f;
+        S[r] = ((en.w > 0 || p.mode == 1) && d < dim && cok) ? stp[(int64_t)d * vdim + c] : 0.f;
     }
     const int64_t HV = (int64_t)p.heads * vdim;
-    for (int t0 = 0; t0 < en.y; t0 += TT) {
+    float run = 1.0f;   // thread d < dimP: product of the entry's gates of row d so far
+    // a thread stages elements i = tid + k * blockDim of the tile's [TT][dimP] q / f and [TT][64] v
+    constexpr int EQ = TT / 2, EV = TT;   // dimP = 32 NG, blockDim = 64 NG
+    float rq[EQ], rf[EQ], rv[EV];
+    auto fetch = [&](int t0) {
         const int nt = min(TT, en.y - t0);
-        __syncthreads();
-        for (int i = tid; i < nt * dimP; i += blockDim.x) {
-            const int tt = i / dimP, d = i % dimP;
+#pragma unroll
+        for (int k = 0; k < EQ; k++) {
+            const int i = tid + k * blockDim.x, tt = i / dimP, d = i % dimP;
+            rq[k] = 0.f;
+            rf[k] = 0.f;
+            if (tt < nt && d < dim) {
+                const float* row = p.proj + (int64_t)(en.x + t0 + tt) * p.ld;
+                rq[k] = row[p.q_col + h * dim + d];
+                rf[k] = row[p.f_col + h * dim + d];
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < EV; k++) {
+            const int i = tid + k * blockDim.x, tt = i >> 6, cc = c0 + (i & 63);
+            rv[k] = (i < TT * 64 && tt < nt && cc < vdim) ? p.proj[(int64_t)(en.x + t0 + tt) * p.ld + p.v_col + h * vdim + cc] : 0.f;
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int k = 0; k < EQ; k++) {
+            const int i = tid + k * blockDim.x, d = i % dimP;
             float qv = 0.f, fv = 1.f;
             if (d < dim) {
-                const float* row = p.proj + (int64_t)(en.x + t0 + tt) * p.ld;
-                const float zq = row[p.q_col + h * dim + d];
-                qv = zq / (1.0f + expf(-zq));
-                const float zf = row[p.f_col + h * dim + d] + p.f_bias[h * dim + d];
+                qv = rq[k] / (1.0f + expf(-rq[k]));
+                const float zf = rf[k] + p.f_bias[h * dim + d];
                 const float l = p.lower[h * dim + d];
                 fv = l + (1.0f - l) * (1.0f / (1.0f + expf(-zf)));
             }
             qs[i] = qv;
             fs[i] = fv;
         }
-        for (int i = tid; i < nt * 64; i += blockDim.x) {
-            const int tt = i >> 6, cc = c0 + (i & 63);
-            vs[i] = cc < vdim ? p.proj[(int64_t)(en.x + t0 + tt) * p.ld + p.v_col + h * vdim + cc] : 0.f;
-        }
-        __syncthreads();
-        for (int tt = 0; tt < nt; tt++) {
-            const float v = vs[tt * 64 + lane];
-            const float* ft = fs + tt * dimP + d0;
-            const float* qt = qs + tt * dimP + d0;
-            float o = 0.f;
 #pragma unroll
-            for (int r = 0; r < SR; r++) {
-                const float f = ft[r];
-                S[r] = fmaf(f, S[r], (1.0f - f) * v);
-                o = fmaf(S[r], qt[r], o);
+        for (int k = 0; k < EV; k++) {
+            const int i = tid + k * blockDim.x;
+            if (i < TT * 64) vs[i] = rv[k];
+        }
+    };
+    fetch(0);
+    for (int t0 = 0; t0 < en.y; t0 += TT) {
+        const int nt = min(TT, en.y - t0);
+        __syncthreads();   // the previous tile's readers are done
+        stage();
+        __syncthreads();
+        if (t0 + TT < en.y) fetch(t0 + TT);
+        if (p.mode == 1 || p.decay) {
+            if (tid < dimP)
+                for (int tt = 0; tt < nt; tt++) {
+                    run *= fs[tt * dimP + tid];
+                    if (p.mode == 1) qs[tt * dimP + tid] *= run;
+                }
+            __syncthreads();
+        }
+        if (p.mode == 0) {
+            for (int tt = 0; tt < nt; tt++) {
+                const float v = vs[tt * 64 + lane];
+                const float4* ft = reinterpret_cast<const float4*>(fs + tt * dimP + d0);
+                const float4* qt = reinterpret_cast<const float4*>(qs + tt * dimP + d0);
+                float o = 0.f;
+#pragma unroll
+                for (int r4 = 0; r4 < SR / 4; r4++) {
+                    const float4 f4 = ft[r4], q4 = qt[r4];
+                    const float f[4] = {f4.x, f4.y, f4.z, f4.w}, q[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        S[4 * r4 + j] = fmaf(f[j], S[4 * r4 + j], (1.0f - f[j]) * v);
+                        o = fmaf(S[4 * r4 + j], q[j], o);
+                    }
+                }
+                op[(tt * NG + grp) * 64 + lane] = o;
             }
-            op[(tt * NG + grp) * 64 + lane] = o;
+        } else {
+            for (int tt = 0; tt < nt; tt++) {
+                const float4* qt = reinterpret_cast<const float4*>(qs + tt * dimP + d0);
+                float o = 0.f;
+#pragma unroll
+                for (int r4 = 0; r4 < SR / 4; r4++) {
+                    const float4 q4 = qt[r4];
+                    o = fmaf(S[4 * r4], q4.x, o);
+                    o = fmaf(S[4 * r4 + 1], q4.y, o);
+                    o = fmaf(S[4 * r4 + 2], q4.z, o);
+                    o = fmaf(S[4 * r4 + 3], q4.w, o);
+                }
+                op[(tt * NG + grp) * 64 + lane] = o;
+            }
         }
         __syncthreads();
         for (int i = tid; i < nt * 64; i += blockDim.x) {
@@ -602,11 +686,13 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(GatedScanP p, int TT, 
             if (c0 + cl < vdim) p.out[(int64_t)(en.x + t0 + tt) * HV + (int64_t)h * vdim + c0 + cl] = o;
         }
     }
+    if (p.mode == 1) return;
 #pragma unroll
     for (int r = 0; r < SR; r++) {
         const int d = d0 + r;
         if (d < dim && cok) stp[(int64_t)d * vdim + c] = S[r];
     }
+    if (p.decay && blockIdx.z == 0 && tid < dim) p.decay[((int64_t)blockIdx.y * p.heads + h) * dim + tid] = run;
 }
 
 int gated_scan(const GatedScanP& p, hipStream_t st) {
@@ -615,36 +701,69 @@ int gated_scan(const GatedScanP& p, hipStream_t st) {
     QIE_REQUIRE(NG <= 16, "gated scan: dim %d above %d", p.dim, 16 * SR);
     const int dimP = NG * SR;
     const int per_tok = (2 * dimP + 64 + NG * 64) * 4;
-    const int TT = std::max(1, std::min(16, 48 * 1024 / per_tok));
-    const size_t shm = (size_t)TT * per_tok;
     dim3 grid((unsigned)p.heads, (unsigned)p.n_entries, (unsigned)((p.vdim + 63) / 64));
-    hipLaunchKernelGGL(gated_scan_kernel, grid, dim3(64 * NG), shm, st, p, TT, dimP);
+    // up to 4 row groups: 256 threads at most, and the register budget that goes with them
+    if (NG <= 4)
+        hipLaunchKernelGGL((gated_scan_kernel<16, 256>), grid, dim3(64 * NG), (size_t)16 * per_tok, st, p, dimP);
+    else if (16 * per_tok <= 60 * 1024)
+        hipLaunchKernelGGL((gated_scan_kernel<16, 1024>), grid, dim3(64 * NG), (size_t)16 * per_tok, st, p, dimP);
+    else
+        hipLaunchKernelGGL((gated_scan_kernel<4, 1024>), grid, dim3(64 * NG), (size_t)4 * per_tok, st, p, dimP);
+    QIE_LAUNCH_CHECK();
+    return 0;
+}
+
+// s_in[c] = the state that enters piece c; one thread per state element walks its entry's pieces.
+__global__ __launch_bounds__(256) void gated_carry_kernel(GatedCarryP p) {
+    const int64_t n = (int64_t)p.heads * p.dim * p.vdim;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int4 sp = p.spans[blockIdx.y];
+    const int64_t hd = i / p.vdim;   // (head, row) of the element: its gate product
+    float* stp = p.state + (int64_t)sp.z * p.slot_stride + p.state_off + i;
+    float S = sp.w > 0 ? *stp : 0.f;
+    for (int c = sp.x; c < sp.x + sp.y; c++) {
+        p.s_in[(int64_t)c * n + i] = S;
+        S = fmaf(p.decay[(int64_t)c * p.heads * p.dim + hd], S, p.s_loc[(int64_t)c * n + i]);
+    }
+    *stp = S;
+}
+int gated_carry(const GatedCarryP& p, hipStream_t st) {
+    QIE_REQUIRE(p.n_spans > 0 && p.s_loc && p.decay && p.s_in && p.state, "gated carry: bad arguments");
+    const int64_t n = (int64_t)p.heads * p.dim * p.vdim;
+    hipLaunchKernelGGL(gated_carry_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)p.n_spans), dim3(256), 0, st, p);
     QIE_LAUNCH_CHECK();
     return 0;
 }
 
 // ------------------------------------------------------------------ per-head norm
-__global__ __launch_bounds__(256) void head_norm_rows_kernel(const float* o, const float* w, float eps, float scale, int heads, int vdim,
-                                                             float* out, uint16_t* out_bf, int64_t ld_out, int out_col) {
+__global__ __launch_bounds__(256) void head_norm_rows_kernel(const float* o, const float* o2, const float* w, float eps, float scale,
+                                                             int heads, int vdim, float* out, uint16_t* out_bf, int64_t ld_out,
+                                                             int out_col) {
     const int64_t t = blockIdx.x;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     for (int h = wave; h < heads; h += 4) {
         const float* x = o + (t * heads + h) * vdim;
+        const float* x2 = o2 ? o2 + (t * heads + h) * vdim : nullptr;
         float ss = 0.f;
-        for (int i = lane; i < vdim; i += 64) ss += x[i] * x[i];
+        for (int i = lane; i < vdim; i += 64) {
+            const float a = x2 ? x[i] + x2[i] : x[i];
+            ss += a * a;
+        }
         ss = wsum(ss);
         const float inv = scale / sqrtf(ss / (float)vdim + eps);
         const int64_t o0 = t * ld_out + out_col + (int64_t)h * vdim;
         for (int i = lane; i < vdim; i += 64) {
-            const float y = x[i] * inv * w[i];
+            const float y = (x2 ? x[i] + x2[i] : x[i]) * inv * w[i];
             out[o0 + i] = y;
             if (out_bf) out_bf[o0 + i] = f2bf(y);
         }
     }
 }
-int head_norm_rows(const float* o, const float* w, float eps, float scale, int heads, int vdim, int T, float* out, uint16_t* out_bf,
-                   int64_t ld_out, int out_col, hipStream_t st) {
-    hipLaunchKernelGGL(head_norm_rows_kernel, dim3(T), dim3(256), 0, st, o, w, eps, scale, heads, vdim, out, out_bf, ld_out, out_col);
+int head_norm_rows(const float* o, const float* o2, const float* w, float eps, float scale, int heads, int vdim, int T, float* out,
+                   uint16_t* out_bf, int64_t ld_out, int out_col, hipStream_t st) {
+    hipLaunchKernelGGL(head_norm_rows_kernel, dim3(T), dim3(256), 0, st, o, o2, w, eps, scale, heads, vdim, out, out_bf, ld_out,
+                       out_col);
     QIE_LAUNCH_CHECK();
     return 0;
 }

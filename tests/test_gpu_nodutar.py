@@ -268,6 +268,25 @@ def test_long_decoding_over_many_pages(model):
     assert rel(feed(m, 0, toks, [9]), m.ref(toks)) < REL32
 
 
+def test_long_portions_scan_in_pieces(model):
+    """Entries of more than 128 rows run the recurrence in pieces of 64 rows side by side and carry the states
+    across afterwards: from a fresh state, from a state left by an earlier portion, beside short entries of other
+    requests, with gates close to one so that every piece's incoming state matters."""
+    m = model([par(size=50, left_scale=0.2, right_scale=1.0, rheads=2, rdim=40, rvdim=70), dist(mlp=None),
+               par(size=7, left_scale=0.2, right_scale=1.0, mlp=None)], seed=55, page_tokens=16, max_ctx=512, loop=(0, 2, 2),
+              tweak=long_memory)
+    toks, other, third = m.tokens(400), m.tokens(30), m.tokens(140)
+    want, want_o, want_t = m.ref(toks), m.ref(other), m.ref(third)
+    assert rel(m.batch.step([(0, toks)], range(400)), want) < REL32                      # 7 pieces from zero
+    a = m.batch.step([(1, toks[:150])], range(150))                                      # 3 pieces, the last one short
+    b1 = m.batch.step([(2, other[:29])], range(29))
+    b = m.batch.step([(1, toks[150:379]), (2, other[29:]), (3, third)], range(229 + 1 + 140))   # pieces from a kept state
+    c = feed(m, 1, toks[379:], [2])
+    assert rel(np.concatenate([a, b[:229], c]), want) < REL32
+    assert rel(np.concatenate([b1, b[229:230]]), want_o) < REL32
+    assert rel(b[230:], want_t) < REL32
+
+
 def test_other_sizes(model):
     """Sizes and constants unlike the shapes above: odd head sizes, one head, many heads, vdim above and below
     dim, a rotary extent of 2, top 3 of 7, different scales per side."""
