@@ -793,7 +793,9 @@ static int enq_gqa_attention(qie_batch* b, int r, int T) {
         const int tiles = (p.heads + 3) / 4 * 4;
         const int64_t waves = (int64_t)s->n_qgroups * p.heads;
         const int max_blocks = (p.mask == QIE_MASK_CAUSAL ? b->max_ctx : std::min(b->max_ctx, p.mask_size)) / 32 + 2;
-        const int S = (int)std::max<int64_t>(1, std::min<int64_t>({2048 / waves, max_blocks / 2, 32}));
+        // (a wave walks its key blocks one after the other, each a trip to memory: prompts of a
+        // few thousand rows leave too few waves to hide them, so their keys are split as well)
+        const int S = (int)std::max<int64_t>(1, std::min<int64_t>({6144 / waves, max_blocks / 4, 32}));
         const int64_t units = (int64_t)s->n_qgroups * tiles * S;
         if (S > 1 && units > s->gpart_cap) {
             hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
@@ -810,7 +812,7 @@ static int enq_gqa_attention(qie_batch* b, int r, int T) {
             QIE_TRY(dmalloc((void**)&s->gpart_ml, (size_t)cap * 16 * 2 * 4));
             s->gpart_cap = cap;
         }
-        lay::GqaAttnMfmaP q{p, s->d_qgroups, s->n_qgroups, S, s->gpart_o, s->gpart_ml};
+        lay::GqaAttnMfmaP q{p, s->d_qgroups, s->n_qgroups, S, s->gpart_o, s->gpart_ml, (p.heads / p.kv_heads) % 4 != 0 ? 1 : 0};
         return lay::gqa_attention_mfma(q, e->stream);
     }
     return lay::gqa_attention(p, e->lm->f32, T, e->stream);

@@ -162,7 +162,7 @@ int gqa_attention(const GqaAttnP& p, bool cache_f32, int T, hipStream_t st);
 // page [kv_heads][vdim][page_tokens], so that 4 keys of one value coordinate are one 8-byte load;
 // page_tokens a multiple of 32), dim a multiple of 32 and vdim of 16, both up to 256.  A wave takes
 // up to 16 (token, head) columns of one slot that share a key head: 16 consecutive tokens of one
-// head, or - for groups of few tokens - the heads of one key head per token.  groups: {first
+// head, or - for groups of few tokens, see pack - the heads of one key head per token.  groups: {first
 // packed row, tokens (<= 16), slot, first position}.  S > 1 splits every wave's keys S ways
 // (decoding: few columns, many keys); the partial sums meet in a second pass.  part_o
 // [groups * tiles * S][16][vdim], part_ml [...][16][2] floats of scratch (tiles = 4 * ceil(heads / 4)).
@@ -172,6 +172,10 @@ struct GqaAttnMfmaP {
     int n_groups, S;
     float* part_o;
     float* part_ml;
+    // 1: groups of few tokens pack the heads of a key head into a wave's columns, every wave loads
+    // its own fragments (head ratios that are no multiple of 4); 0: one head per wave, the four
+    // waves of a workgroup share their key head's tiles through LDS (ratios that are)
+    int pack;
 };
 bool gqa_attention_mfma_fits(int dim, int vdim, int page_tokens);
 int gqa_attention_mfma(const GqaAttnMfmaP& p, hipStream_t st);

@@ -343,19 +343,27 @@ __device__ __forceinline__ void gqa_store(const GqaAttnP& a, const gf32x4_t* acc
     }
 }
 
-template <int DK, int DV>
+// SHARE: the four waves of a workgroup are four heads of one key head (heads / kv_heads a
+// multiple of 4, one head per wave whatever the group's size): every 32-key K tile and V^T tile
+// is brought to LDS once per workgroup (next tile in registers meanwhile) and each wave takes
+// its fragments from there - a quarter of the cache traffic of four waves loading for themselves.
+template <int DK, int DV, bool SHARE>
 __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(GqaAttnMfmaP P) {
     const GqaAttnP& a = P.a;
     constexpr int dim = 32 * DK, vdim = 16 * DV;
+    constexpr int KROW = dim + 8, VROW = 32 + 8;   // LDS rows padded by 16 bytes
+    __shared__ __align__(16) uint16_t lk[SHARE ? 32 * KROW : 8];
+    __shared__ __align__(16) uint16_t lv[SHARE ? vdim * VROW : 8];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 4, n = lane & 15;
     const int4 grp = P.groups[blockIdx.x];
     const int n_tok = grp.y, slot = grp.z, pos0 = grp.w;
     const int H = a.heads, G = a.kv_heads;
-    const int hpt = heads_per_token(n_tok, H, G);
-    const int tile = blockIdx.y * 4 + wave, h0 = tile * hpt;
-    if (h0 >= H) return;
+    const int hpt = SHARE ? 1 : heads_per_token(n_tok, H, G);
+    const int tile = blockIdx.y * 4 + wave, h0 = SHARE ? min(tile, H - 1) : tile * hpt;
+    const bool active = SHARE ? tile < H : true;
+    if (!SHARE && h0 >= H) return;
     const int tI = n / hpt, hh = h0 + n % hpt;
-    const bool valid = tI < n_tok;
+    const bool valid = active && tI < n_tok;
     const int tC = valid ? tI : n_tok - 1;
     const int qpos = pos0 + tC, row = grp.x + tC;
     const int kvh = h0 / (H / G);
@@ -399,21 +407,68 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(GqaAttnMfmaP P) {
             for (int ks = 0; ks < DK; ks++) dst[tt][ks] = *reinterpret_cast<const uint4*>(kr + 32 * ks);
         }
     };
-    if (bs < be) load_k(bs, kf);
+    // SHARE: a thread's 16-byte pieces of the workgroup's tiles (K: 32 keys x dim, V^T: vdim x 32 keys)
+    constexpr int NKP = (32 * dim / 8 + 255) / 256, NVP = (vdim * 4 + 255) / 256;
+    uint4 gk[NKP], gv[NVP];
+    auto fetch_tiles = [&](int kb) {
+        const int key0 = kb << 5;
+        const int64_t pb = (int64_t)tab[key0 / PT] * a.cache.page_stride;
+        const int tok0 = key0 % PT;
+#pragma unroll
+        for (int k = 0; k < NKP; k++) {
+            const int c = (int)threadIdx.x + 256 * k, key = c / (dim / 8), part = c % (dim / 8);
+            if (c < 32 * dim / 8) gk[k] = *reinterpret_cast<const uint4*>(pool + pb + a.k_off + ((int64_t)(tok0 + key) * G + kvh) * dim + part * 8);
+        }
+#pragma unroll
+        for (int k = 0; k < NVP; k++) {
+            const int c = (int)threadIdx.x + 256 * k, r = c >> 2, part = c & 3;
+            if (c < vdim * 4) gv[k] = *reinterpret_cast<const uint4*>(pool + pb + a.v_off + ((int64_t)kvh * vdim + r) * PT + tok0 + part * 8);
+        }
+    };
+    auto store_tiles = [&]() {
+#pragma unroll
+        for (int k = 0; k < NKP; k++) {
+            const int c = (int)threadIdx.x + 256 * k, key = c / (dim / 8), part = c % (dim / 8);
+            if (c < 32 * dim / 8) *reinterpret_cast<uint4*>(lk + key * KROW + part * 8) = gk[k];
+        }
+#pragma unroll
+        for (int k = 0; k < NVP; k++) {
+            const int c = (int)threadIdx.x + 256 * k, r = c >> 2, part = c & 3;
+            if (c < vdim * 4) *reinterpret_cast<uint4*>(lv + r * VROW + part * 8) = gv[k];
+        }
+    };
+    if (bs < be) {
+        if (SHARE) fetch_tiles(bs);
+        else load_k(bs, kf);
+    }
     for (int kb = bs; kb < be; kb++) {
         const int key0 = kb << 5;
         const int64_t pb = (int64_t)tab[key0 / PT] * a.cache.page_stride;
         const int tok0 = key0 % PT;
         uint2 vf[DV][2];
-        {
+        if (SHARE) {
+            __syncthreads();   // the previous tiles have been read
+            store_tiles();
+            __syncthreads();
+            if (kb + 1 < be) fetch_tiles(kb + 1);
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                for (int ks = 0; ks < DK; ks++) kf[tt][ks] = *reinterpret_cast<const uint4*>(lk + (16 * tt + n) * KROW + 32 * ks + 8 * g);
+#pragma unroll
+            for (int dv = 0; dv < DV; dv++) {
+                vf[dv][0] = *reinterpret_cast<const uint2*>(lv + (16 * dv + n) * VROW + 4 * g);
+                vf[dv][1] = *reinterpret_cast<const uint2*>(lv + (16 * dv + n) * VROW + 16 + 4 * g);
+            }
+        } else {
             const uint16_t* vr = pool + pb + a.v_off + ((int64_t)kvh * vdim + n) * PT + tok0 + 4 * g;
 #pragma unroll
             for (int dv = 0; dv < DV; dv++) {
                 vf[dv][0] = *reinterpret_cast<const uint2*>(vr + (int64_t)16 * dv * PT);
                 vf[dv][1] = *reinterpret_cast<const uint2*>(vr + (int64_t)16 * dv * PT + 16);
             }
+            if (kb + 1 < be) load_k(kb + 1, kn);
         }
-        if (kb + 1 < be) load_k(kb + 1, kn);
         gf32x4_t sacc[2];
 #pragma unroll
         for (int tt = 0; tt < 2; tt++) {
@@ -455,11 +510,14 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(GqaAttnMfmaP P) {
             for (int j = 0; j < 4; j++) acc[dv][j] *= alpha;
             acc[dv] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(gbf16x8_t, vu), pf, acc[dv], 0, 0, 0);
         }
+        if (!SHARE) {
 #pragma unroll
-        for (int tt = 0; tt < 2; tt++)
+            for (int tt = 0; tt < 2; tt++)
 #pragma unroll
-            for (int ks = 0; ks < DK; ks++) kf[tt][ks] = kn[tt][ks];
+                for (int ks = 0; ks < DK; ks++) kf[tt][ks] = kn[tt][ks];
+        }
     }
+    if (!active) return;
     if (S == 1) {
         if (valid) gqa_store<DV>(a, acc, 1.0f / l_run, row, hh, qpos, g);
         return;
@@ -482,28 +540,40 @@ __global__ __launch_bounds__(256) void gqa_attn_combine_kernel(GqaAttnMfmaP P, i
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 4, n = lane & 15;
     const int4 grp = P.groups[blockIdx.x];
     const int n_tok = grp.y, pos0 = grp.w;
-    const int hpt = heads_per_token(n_tok, a.heads, a.kv_heads);
+    const int hpt = P.pack ? heads_per_token(n_tok, a.heads, a.kv_heads) : 1;
     const int tile = blockIdx.y * 4 + wave, h0 = tile * hpt;
     if (h0 >= a.heads) return;
     const int tI = n / hpt, hh = h0 + n % hpt;
     if (tI >= n_tok) return;
     const int64_t u0 = ((int64_t)blockIdx.x * tiles + tile) * P.S;
+    const float* ml = P.part_ml + (u0 * 16 + n) * 2;          // part z at ml + 32 z
     float M = -1e30f;
-    for (int z = 0; z < P.S; z++) M = fmaxf(M, P.part_ml[((u0 + z) * 16 + n) * 2]);
+    for (int z = 0; z < P.S; z++) M = fmaxf(M, ml[32 * z]);
     float L = 0.f;
     gf32x4_t acc[DV];
 #pragma unroll
     for (int dv = 0; dv < DV; dv++) acc[dv] = gf32x4_t{0.f, 0.f, 0.f, 0.f};
-    for (int z = 0; z < P.S; z++) {
-        const float l = P.part_ml[((u0 + z) * 16 + n) * 2 + 1];
-        if (l == 0.f) continue;   // this part saw no key of the column
-        const float w = expf(P.part_ml[((u0 + z) * 16 + n) * 2] - M);
-        L += l * w;
-        const float* po = P.part_o + ((u0 + z) * 16 + n) * vdim + 4 * g;
+    // two parts a turn, every load of the turn issued before its first use; a part that saw no key
+    // of the column has l = 0 and zero sums
+    for (int z0 = 0; z0 < P.S; z0 += 2) {
+        const int z1 = min(z0 + 1, P.S - 1);
+        const float w0 = ml[32 * z0 + 1] == 0.f ? 0.f : __expf(ml[32 * z0] - M);
+        const float w1 = (z0 + 1 >= P.S || ml[32 * z1 + 1] == 0.f) ? 0.f : __expf(ml[32 * z1] - M);
+        L += ml[32 * z0 + 1] * w0 + ml[32 * z1 + 1] * w1;
+        const float* p0 = P.part_o + ((u0 + z0) * 16 + n) * vdim + 4 * g;
+        const float* p1 = P.part_o + ((u0 + z1) * 16 + n) * vdim + 4 * g;
+        float4 o0[DV], o1[DV];
 #pragma unroll
         for (int dv = 0; dv < DV; dv++) {
-            const float4 o = *reinterpret_cast<const float4*>(po + 16 * dv);
-            acc[dv][0] += o.x * w; acc[dv][1] += o.y * w; acc[dv][2] += o.z * w; acc[dv][3] += o.w * w;
+            o0[dv] = *reinterpret_cast<const float4*>(p0 + 16 * dv);
+            o1[dv] = *reinterpret_cast<const float4*>(p1 + 16 * dv);
+        }
+#pragma unroll
+        for (int dv = 0; dv < DV; dv++) {
+            acc[dv][0] += o0[dv].x * w0 + o1[dv].x * w1;
+            acc[dv][1] += o0[dv].y * w0 + o1[dv].y * w1;
+            acc[dv][2] += o0[dv].z * w0 + o1[dv].z * w1;
+            acc[dv][3] += o0[dv].w * w0 + o1[dv].w * w1;
         }
     }
     gqa_store<DV>(a, acc, 1.0f / L, grp.x + tI, hh, pos0 + tI, g);
@@ -514,27 +584,21 @@ bool gqa_attention_mfma_fits(int dim, int vdim, int page_tokens) {
     return one_of(dim, 32) && one_of(vdim, 32) && page_tokens % 32 == 0;
 }
 
+template <int DK, int DV>
+static void gqa_mfma_launch2(const GqaAttnMfmaP& p, dim3 grid, hipStream_t st) {
+    if (p.pack)
+        hipLaunchKernelGGL((gqa_attn_mfma_kernel<DK, DV, false>), grid, dim3(256), 0, st, p);
+    else
+        hipLaunchKernelGGL((gqa_attn_mfma_kernel<DK, DV, true>), grid, dim3(256), 0, st, p);
+    if (p.S > 1) hipLaunchKernelGGL(gqa_attn_combine_kernel<DV>, dim3(grid.x, grid.y, 1), dim3(256), 0, st, p, (int)grid.y * 4);
+}
 template <int DK>
 static int gqa_mfma_launch(const GqaAttnMfmaP& p, dim3 grid, hipStream_t st) {
-    const int tiles = (int)grid.y * 4;
-    dim3 cg(grid.x, grid.y, 1);
     switch (p.a.vdim / 32) {
-        case 1:
-            hipLaunchKernelGGL((gqa_attn_mfma_kernel<DK, 2>), grid, dim3(256), 0, st, p);
-            if (p.S > 1) hipLaunchKernelGGL(gqa_attn_combine_kernel<2>, cg, dim3(256), 0, st, p, tiles);
-            break;
-        case 2:
-            hipLaunchKernelGGL((gqa_attn_mfma_kernel<DK, 4>), grid, dim3(256), 0, st, p);
-            if (p.S > 1) hipLaunchKernelGGL(gqa_attn_combine_kernel<4>, cg, dim3(256), 0, st, p, tiles);
-            break;
-        case 4:
-            hipLaunchKernelGGL((gqa_attn_mfma_kernel<DK, 8>), grid, dim3(256), 0, st, p);
-            if (p.S > 1) hipLaunchKernelGGL(gqa_attn_combine_kernel<8>, cg, dim3(256), 0, st, p, tiles);
-            break;
-        default:
-            hipLaunchKernelGGL((gqa_attn_mfma_kernel<DK, 16>), grid, dim3(256), 0, st, p);
-            if (p.S > 1) hipLaunchKernelGGL(gqa_attn_combine_kernel<16>, cg, dim3(256), 0, st, p, tiles);
-            break;
+        case 1: gqa_mfma_launch2<DK, 2>(p, grid, st); break;
+        case 2: gqa_mfma_launch2<DK, 4>(p, grid, st); break;
+        case 4: gqa_mfma_launch2<DK, 8>(p, grid, st); break;
+        default: gqa_mfma_launch2<DK, 16>(p, grid, st); break;
     }
     QIE_LAUNCH_CHECK();
     return 0;
@@ -546,6 +610,7 @@ int gqa_attention_mfma(const GqaAttnMfmaP& p, hipStream_t st) {
                 "gqa attention: sizes %d / %d, pages of %d tokens do not fit the matrix-core form", a.dim, a.vdim, a.cache.page_tokens);
     QIE_REQUIRE(p.n_groups > 0 && p.S >= 1 && (p.S == 1 || (p.part_o && p.part_ml)), "gqa attention: bad launch");
     QIE_REQUIRE(a.heads % a.kv_heads == 0, "gqa attention: %d query heads over %d key heads", a.heads, a.kv_heads);
+    QIE_REQUIRE(p.pack == ((a.heads / a.kv_heads) % 4 != 0), "gqa attention: packing goes with head ratios that are no multiple of 4");
     dim3 grid((unsigned)p.n_groups, (unsigned)((a.heads + 3) / 4), (unsigned)p.S);
     switch (a.dim / 32) {
         case 1: return gqa_mfma_launch<1>(p, grid, st);
