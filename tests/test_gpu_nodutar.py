@@ -305,8 +305,9 @@ def test_bf16_matrix_shapes(model, hd, size, page):
     """Sizes that take the bf16 matrix kernels (pages of 32 or more tokens: attention on the matrix cores over
     transposed value rows, key splits while decoding; pages of 16: the plain attention): whole prompts, portions
     and single tokens against the oracle, beside another request, with more than 256 routed rows in one step."""
-    layers = [par(heads=4, kv_heads=2, dim=hd, vdim=hd, rot_dims=hd // 2, size=size, scale=0.5, rheads=2, rdim=32, rvdim=64,
-                  mlp=("moe", 32, 4, 2)),
+    # pages of 64: 8 heads over 2 key heads (the four waves of a workgroup share their key head's tiles); else 4 over 2
+    layers = [par(heads=8 if page == 64 else 4, kv_heads=2, dim=hd, vdim=hd, rot_dims=hd // 2, size=size, scale=0.5, rheads=2, rdim=32,
+                  rvdim=64, mlp=("moe", 32, 4, 2)),
               dist(heads=4, kv_heads=1, dim=hd, scale=1.0, mlp=("moe", 96, 4, 2))]
     m = model(layers, seed=hd, vocab=160, width=64, dtype="bfloat16", page_tokens=page, max_ctx=512, loop=(0, 1, 2))
     toks = m.tokens(150)
