@@ -201,7 +201,7 @@ def nodutar_model(S, size):
     par = {"type": "parallel", "mlp": moe, "mixer": {
         "left": {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "mask": {"size": blk}, "rot": {"base": 10000.0, "dims": rot},
                  "scale": hd ** -0.5},
-        "right": {"heads": RH, "dim": rd, "vdim": rv}, "left_scale": 0.8, "right_scale": 0.5}}
+        "right": {"heads": RH, "dim": rd, "vdim": rv}, "left_scale": 1.0, "right_scale": 1.0}}
     att = {"type": "attention", "mlp": moe, "mixer": {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5 * 4}}
     cfg = {"architecture": "Nodutar", "layers": [par, att, par, att], "norm": {"eps": 1e-6}, "vocab": V, "width": W}
     spec = S.spec_from_config(cfg, name=f"nodutar-{size}")

@@ -795,7 +795,8 @@ static int enq_gqa_attention(qie_batch* b, int r, int T) {
         const int max_blocks = (p.mask == QIE_MASK_CAUSAL ? b->max_ctx : std::min(b->max_ctx, p.mask_size)) / 32 + 2;
         // (a wave walks its key blocks one after the other, each a trip to memory: prompts of a
         // few thousand rows leave too few waves to hide them, so their keys are split as well)
-        const int S = (int)std::max<int64_t>(1, std::min<int64_t>({6144 / waves, max_blocks / 4, 32}));
+        static const int split_waves = dev_env("QIE_GQA_SPLIT_WAVES", 6144);   // dev A/B knob: waves a launch aims for
+        const int S = (int)std::max<int64_t>(1, std::min<int64_t>({split_waves / waves, max_blocks / 4, 32}));
         const int64_t units = (int64_t)s->n_qgroups * tiles * S;
         if (S > 1 && units > s->gpart_cap) {
             hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
